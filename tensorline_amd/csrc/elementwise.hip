@@ -1,0 +1,225 @@
+// Row-wise and element-wise kernels: embedding gather, residual add + RMSNorm, rotary position
+// encoding fused with the write into the paged cache, SiLU-multiply.
+//
+// The residual stream is float in every mode; the kernels that read or write activations take
+// the storage type (float or bfloat16) as a template argument and compute in float.
+#include "common.h"
+
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+// ---- error reporting -----------------------------------------------------------------------
+static thread_local char g_tl_error[512] = "";
+
+int tl_fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_tl_error, sizeof(g_tl_error), fmt, ap);
+    va_end(ap);
+    return 1;
+}
+
+extern "C" const char* tl_last_error() { return g_tl_error; }
+
+extern "C" int tl_abi_version() { return 1; }
+
+// ---- embedding gather ----------------------------------------------------------------------
+// x[t, :] = float(table[ids[t], :]).  An id outside [0, V) gives a row of NaN instead of a fault;
+// callers validate ids on the host.
+template <typename T>
+__global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
+                             float* __restrict__ x, int H, int V) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* xr = x + (size_t)t * H;
+    if (id < 0 || id >= V) {
+        for (int c = threadIdx.x; c < H; c += blockDim.x) xr[c] = NAN;
+        return;
+    }
+    const T* row = table + (size_t)id * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) xr[c] = tl_to_float(row[c]);
+}
+
+extern "C" int tl_embed(const int32_t* ids, const void* table, int table_dtype, float* x, int T, int H, int V,
+                        hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && H > 0 && V > 0, "tl_embed: bad sizes T=%d H=%d V=%d", T, H, V);
+    if (T == 0) return 0;
+    dim3 grid(T), block(256);
+    if (table_dtype == TL_F32)
+        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, (const float*)table, x, H, V);
+    else if (table_dtype == TL_BF16)
+        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, (const bf16_t*)table, x, H, V);
+    else
+        return tl_fail("tl_embed: unknown dtype %d", table_dtype);
+    TL_CHECK_LAUNCH("tl_embed");
+    return 0;
+}
+
+// ---- residual add + RMSNorm ----------------------------------------------------------------
+// Without `rows`: x[r] += residual[r] (written back, float), out[r] = x[r] * rstd * w.
+// With `rows`:    out[r] = norm(x[rows[r]] + residual[rows[r]]); x is left as it is.
+// The sum, the mean of squares and the scaling are float (reference: tensorline/fused.py:19-32).
+template <typename R, typename O, bool HAS_RES, bool HAS_ROWS>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const R* __restrict__ res, const float* __restrict__ w,
+                                   O* __restrict__ out, const int32_t* __restrict__ rows, int H, float eps) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const size_t src = HAS_ROWS ? (size_t)rows[r] : (size_t)r;
+    float* xr = x + src * H;
+    const R* rr = HAS_RES ? res + src * H : nullptr;
+    O* orow = out + (size_t)r * H;
+
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = xr[c];
+        if (HAS_RES) {
+            v += tl_to_float(rr[c]);
+            if (!HAS_ROWS) xr[c] = v;
+        }
+        ss += v * v;
+    }
+    ss = tl_block_sum(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = xr[c];
+        if (HAS_RES && HAS_ROWS) v += tl_to_float(rr[c]);
+        orow[c] = tl_from_float<O>(v * rstd * w[c]);
+    }
+}
+
+template <typename R, typename O>
+static void launch_add_rmsnorm(float* x, const R* res, const float* w, O* out, const int32_t* rows, int n_rows,
+                               int H, float eps, hipStream_t stream) {
+    dim3 grid(n_rows), block(H >= 2048 ? 512 : 256);
+    if (res && rows)
+        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, true, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+    else if (res)
+        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, true, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+    else if (rows)
+        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, false, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+    else
+        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, false, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+}
+
+extern "C" int tl_add_rmsnorm(float* x, const void* residual, int res_dtype, const float* w, void* out, int out_dtype,
+                              const int32_t* rows, int n_rows, int H, float eps, hipStream_t stream) {
+    TL_CHECK_ARG(n_rows >= 0 && H > 0, "tl_add_rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+    TL_CHECK_ARG(eps >= 0.f, "tl_add_rmsnorm: eps must be >= 0");
+    if (n_rows == 0) return 0;
+    if (!residual) res_dtype = TL_F32;
+#define TL_NORM_CASE(RD, RT, OD, OT)                                                                     \
+    if (res_dtype == RD && out_dtype == OD) {                                                            \
+        launch_add_rmsnorm<RT, OT>(x, (const RT*)residual, w, (OT*)out, rows, n_rows, H, eps, stream);  \
+        TL_CHECK_LAUNCH("tl_add_rmsnorm");                                                               \
+        return 0;                                                                                        \
+    }
+    TL_NORM_CASE(TL_F32, float, TL_F32, float)
+    TL_NORM_CASE(TL_F32, float, TL_BF16, bf16_t)
+    TL_NORM_CASE(TL_BF16, bf16_t, TL_F32, float)
+    TL_NORM_CASE(TL_BF16, bf16_t, TL_BF16, bf16_t)
+#undef TL_NORM_CASE
+    return tl_fail("tl_add_rmsnorm: unknown dtypes residual=%d out=%d", res_dtype, out_dtype);
+}
+
+// ---- rotary position encoding + cache write ------------------------------------------------
+// qkv: [T, (nq + 2 nkv) * d] as the fused projection leaves it.  Query heads are rotated in place;
+// key heads are rotated and written to k_cache at the token's slot; value heads are copied to
+// v_cache.  Rotate-half layout over the first `rot` dims of a head (reference: fused.py:34-51):
+//   out[i]         = a*cos(theta_i) - b*sin(theta_i)       a = x[i], b = x[i + rot/2]
+//   out[i + rot/2] = b*cos(theta_i) + a*sin(theta_i)       theta_i = pos * inv_freq[i]
+// The angle, sine and cosine are float.  A negative slot skips the cache write of that token.
+// Caches are [pages, page, nkv, d], addressed here as [slot, nkv, d].
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict__ pos,
+                                  const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                  const int32_t* __restrict__ slots, int nq, int nkv, int d, int rot, int write_kv) {
+    const int t = blockIdx.x;
+    const int half = rot / 2;
+    const float p = (float)pos[t];
+    const int slot = write_kv ? slots[t] : -1;
+    T* row = qkv + (size_t)t * (nq + 2 * nkv) * d;
+    const int nrot = nq + nkv;  // heads that are rotated: q then k
+    // rotated pairs
+    for (int idx = threadIdx.x; idx < nrot * half; idx += blockDim.x) {
+        const int h = idx / half, i = idx - h * half;
+        float sn, cs;
+        sincosf(p * inv_freq[i], &sn, &cs);
+        T* hp = row + (size_t)h * d;
+        const float a = tl_to_float(hp[i]), b = tl_to_float(hp[i + half]);
+        const T o1 = tl_from_float<T>(a * cs - b * sn);
+        const T o2 = tl_from_float<T>(b * cs + a * sn);
+        if (h < nq) {
+            hp[i] = o1;
+            hp[i + half] = o2;
+        } else if (slot >= 0) {
+            T* kp = k_cache + ((size_t)slot * nkv + (h - nq)) * d;
+            kp[i] = o1;
+            kp[i + half] = o2;
+        }
+    }
+    if (slot < 0) return;
+    // key dims beyond the rotated part pass through
+    const int tail = d - rot;
+    for (int idx = threadIdx.x; idx < nkv * tail; idx += blockDim.x) {
+        const int h = idx / tail, i = rot + (idx - h * tail);
+        k_cache[((size_t)slot * nkv + h) * d + i] = row[(size_t)(nq + h) * d + i];
+    }
+    // values
+    const T* vrow = row + (size_t)(nq + nkv) * d;
+    T* vdst = v_cache + (size_t)slot * nkv * d;
+    for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x) vdst[idx] = vrow[idx];
+}
+
+extern "C" int tl_rope_store(void* qkv, int dtype, const int32_t* pos, const float* inv_freq, void* k_cache,
+                             void* v_cache, const int32_t* slots, int T, int nq, int nkv, int d, int rot,
+                             int write_kv, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && nq > 0 && nkv >= 0 && d > 0, "tl_rope_store: bad sizes T=%d nq=%d nkv=%d d=%d", T, nq, nkv, d);
+    TL_CHECK_ARG(rot >= 0 && rot <= d && rot % 2 == 0, "tl_rope_store: rotary width %d must be even and <= head size %d", rot, d);
+    TL_CHECK_ARG(!write_kv || (k_cache && v_cache && slots), "tl_rope_store: cache write asked for without a cache");
+    if (T == 0) return 0;
+    dim3 grid(T), block(256);
+    if (dtype == TL_F32)
+        hipLaunchKernelGGL(rope_store_kernel<float>, grid, block, 0, stream, (float*)qkv, pos, inv_freq,
+                           (float*)k_cache, (float*)v_cache, slots, nq, nkv, d, rot, write_kv);
+    else if (dtype == TL_BF16)
+        hipLaunchKernelGGL(rope_store_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, pos, inv_freq,
+                           (bf16_t*)k_cache, (bf16_t*)v_cache, slots, nq, nkv, d, rot, write_kv);
+    else
+        return tl_fail("tl_rope_store: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("tl_rope_store");
+    return 0;
+}
+
+// ---- SiLU(gate) * up ------------------------------------------------------------------------
+// gu: [T, 2 I] with the gate in the first I columns and the up projection in the last I.
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I) {
+    const int t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= I) return;
+    const T* row = gu + (size_t)t * 2 * I;
+    const float g = tl_to_float(row[i]), u = tl_to_float(row[I + i]);
+    out[(size_t)t * I + i] = tl_from_float<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int tl_silu_mul(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && I > 0, "tl_silu_mul: bad sizes T=%d I=%d", T, I);
+    TL_CHECK_ARG(T <= 65535 * 64, "tl_silu_mul: too many rows %d", T);
+    if (T == 0) return 0;
+    // grid.y is limited to 65535: rows beyond that are covered by repeated launches.
+    for (int t0 = 0; t0 < T; t0 += 65535) {
+        const int tn = (T - t0 < 65535) ? T - t0 : 65535;
+        dim3 grid(tl_ceil_div(I, 256), tn), block(256);
+        if (dtype == TL_F32)
+            hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu + (size_t)t0 * 2 * I,
+                               (float*)out + (size_t)t0 * I, I);
+        else if (dtype == TL_BF16)
+            hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu + (size_t)t0 * 2 * I,
+                               (bf16_t*)out + (size_t)t0 * I, I);
+        else
+            return tl_fail("tl_silu_mul: unknown dtype %d", dtype);
+    }
+    TL_CHECK_LAUNCH("tl_silu_mul");
+    return 0;
+}

@@ -1,0 +1,84 @@
+"""The step function: runs exactly the tokens it is given, as one batch, from the cache.
+
+``ModelRunner.step(entries)`` takes any mix of prompt portions and single decoded tokens
+(:class:`tensorline_amd.engine.batch.StepEntry`), writes their keys and values into the pages the
+cache manager holds for each request, and returns float32 logits at the wanted places, in the
+order of the entries and of their ``want`` lists (reference: ``PagedModel.forward``,
+tensorline/paged.py:190-287).  Generation, trace replay and the benchmark all call this one
+function.
+"""
+from __future__ import annotations
+
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from tensorline_amd.cache.manager import CacheManager
+from tensorline_amd.engine.batch import LayerCache, PackedBatch, StepContext, StepEntry, pack_batch
+from tensorline_amd.models.decoder import DecoderModel
+
+
+class ModelRunner:
+    def __init__(self, model: DecoderModel, cache: CacheManager):
+        self.model = model
+        self.cache = cache
+        self.device = model.device
+        self._host: torch.Tensor | None = None       # pinned staging for the step's metadata
+        self._dev: torch.Tensor | None = None
+        self.steps = 0
+
+    # ---- metadata ------------------------------------------------------------------------
+    def _upload(self, data: np.ndarray) -> torch.Tensor:
+        n = int(data.size)
+        if self._dev is None or self._dev.numel() < n:
+            cap = max(4096, 1 << (max(n, 1) - 1).bit_length())
+            pin = torch.device(self.device).type == "cuda"
+            self._host = torch.empty(cap, dtype=torch.int32, pin_memory=pin)
+            self._dev = torch.empty(cap, dtype=torch.int32, device=self.device)
+        self._host[:n].numpy()[:] = data
+        # A blocking copy: the staging buffer is free for the next step when this returns.
+        self._dev[:n].copy_(self._host[:n], non_blocking=False)
+        return self._dev
+
+    def pack(self, entries: Sequence[StepEntry], pad_seqs: int = 0, pad_nb: Sequence[int] | None = None) -> PackedBatch:
+        cache = self.cache
+        ngroups = len(cache.groups)
+        tables = [[cache.table(e.rid, g) for g in range(ngroups)] for e in entries]
+        slots = [cache.state_slot(e.rid) for e in entries]
+        return pack_batch(entries, tables, slots, cache.page_size, ngroups, cache.scratch_page,
+                          self.model.vocab_size, pad_seqs=pad_seqs, pad_nb=pad_nb, scratch_slot=cache.scratch_slot)
+
+    def context(self, packed: PackedBatch, dev: torch.Tensor) -> tuple[StepContext, list[LayerCache]]:
+        def view(name: str) -> torch.Tensor:
+            off, n = packed.offsets[name]
+            return dev[off:off + n]
+
+        ctx = StepContext(
+            num_tokens=packed.T, num_seqs=packed.S, ids=view("ids"), pos=view("pos"),
+            seq_of_token=view("seq_of_token"), q_start=view("q_start"), ctx_start=view("ctx_start"),
+            state_slots=view("state_slots"), logit_rows=view("logit_rows"), attention_plan=packed.plan,
+            host_q_start=packed.host_q_start, host_ctx_start=packed.host_ctx_start,
+            host_state_slots=packed.host_state_slots)
+        cache = self.cache
+        g_slots = [view(f"slots{g}") for g in range(len(cache.groups))]
+        g_tables = [view(f"tables{g}").view(packed.S, packed.group_nb[g]) for g in range(len(cache.groups))]
+        views: list[LayerCache] = []
+        for i in range(len(self.model.schedule)):
+            g = cache.group_of_entry[i]
+            k, v = cache.storage(i)
+            views.append(LayerCache(
+                k=k, v=v, slots=g_slots[g] if g is not None else None,
+                tables=g_tables[g] if g is not None else None,
+                write=cache.owns_storage(i), state=cache.state.get(i)))
+        return ctx, views
+
+    # ---- one step ------------------------------------------------------------------------
+    @torch.inference_mode()
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Logits [number of wanted places, vocab] in float32."""
+        packed = self.pack(entries)
+        dev = self._upload(packed.data)
+        ctx, views = self.context(packed, dev)
+        self.steps += 1
+        return self.model.forward(ctx, views)

@@ -1,0 +1,266 @@
+"""Python entry to the HIP kernels.
+
+Each function checks shapes, dtypes, devices and layout on the host, then calls one C entry
+point of ``libtensorline_hip.so`` on torch's current stream.  There is no fallback: a missing
+library, a tensor that is not on the GPU or a size a kernel does not take raises an error.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+
+import torch
+
+from tensorline_amd.ops import build as _build
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_lib = None
+_lib_lock = threading.Lock()
+
+
+def library() -> ctypes.CDLL:
+    """The loaded kernel library; built at the first call if no built one matches the sources."""
+    global _lib
+    if _lib is None:
+        with _lib_lock:
+            if _lib is None:
+                path = _build.ensure_built()
+                try:
+                    lib = ctypes.CDLL(path)
+                except OSError as e:
+                    raise KernelError(f"cannot load the HIP kernel library {path}: {e}") from e
+                lib.tl_last_error.restype = ctypes.c_char_p
+                _lib = lib
+    return _lib
+
+
+def library_path() -> str | None:
+    return _build.find_built()
+
+
+def require_gpu(device) -> torch.device:
+    """The engine runs on a ROCm GPU only."""
+    dev = torch.device(device)
+    if dev.type != "cuda":
+        raise KernelError(f"tensorline_amd runs on a ROCm GPU (device 'cuda:N'), not on {dev}")
+    if not torch.cuda.is_available():
+        raise KernelError("no ROCm GPU is visible to torch: the engine has no CPU path")
+    library()
+    return dev
+
+
+def _call(name: str, *args) -> None:
+    fn = getattr(library(), name)
+    rc = fn(*args)
+    if rc != 0:
+        raise KernelError(library().tl_last_error().decode("utf-8", "replace"))
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: torch.Tensor | None) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"{what}: dtype {t.dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _on_gpu(*tensors: torch.Tensor | None) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        _check(t.is_cuda, f"tensor of shape {tuple(t.shape)} is on {t.device}, not on the GPU")
+        dev = dev or t.device
+        _check(t.device == dev, "tensors are on different devices")
+
+
+def _i32(t: torch.Tensor, what: str, n: int | None = None) -> None:
+    _check(t.dtype == torch.int32 and t.is_contiguous(), f"{what} must be a contiguous int32 tensor")
+    if n is not None:
+        _check(t.numel() >= n, f"{what} has {t.numel()} entries, {n} are needed")
+
+
+# ---------------------------------------------------------------------------------------------
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """x[t] = float(table[ids[t]]); the residual stream is float32 in every mode."""
+    _on_gpu(ids, table, out)
+    _i32(ids, "ids")
+    _check(table.dim() == 2 and table.is_contiguous(), "embedding table must be a contiguous [V, H] matrix")
+    T, (V, H) = ids.numel(), table.shape
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.float32, device=table.device)
+    _check(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H), "embed: bad output")
+    _call("tl_embed", _ptr(ids), _ptr(table), _code(table, "embed"), _ptr(out), T, H, V, _stream())
+    return out
+
+
+def add_rmsnorm(x: torch.Tensor, residual: torch.Tensor | None, weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: torch.Tensor | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor:
+    """Without ``rows``: ``x += residual`` in place (float32), returns ``RMSNorm(x) * weight``.
+    With ``rows``: returns the norm of ``x[rows] + residual[rows]`` and leaves ``x`` alone."""
+    _on_gpu(x, residual, weight, rows, out)
+    _check(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "add_rmsnorm: x must be contiguous float32 [T, H]")
+    T, H = x.shape
+    _check(weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() == H,
+           f"add_rmsnorm: weight must be float32 of {H} entries")
+    res_code = F32
+    if residual is not None:
+        _check(residual.is_contiguous() and tuple(residual.shape) == (T, H), "add_rmsnorm: residual must match x")
+        res_code = _code(residual, "add_rmsnorm residual")
+    n = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.numel()
+    if out is None:
+        out = torch.empty(n, H, dtype=out_dtype, device=x.device)
+    _check(out.dtype == out_dtype and out.is_contiguous() and tuple(out.shape) == (n, H), "add_rmsnorm: bad output")
+    _call("tl_add_rmsnorm", _ptr(x), _ptr(residual), res_code, _ptr(weight), _ptr(out), _code(out, "add_rmsnorm out"),
+          _ptr(rows), n, H, ctypes.c_float(eps), _stream())
+    return out
+
+
+def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+           out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``a @ weight.T + bias``: a [M, K] (rows may be strided), weight [N, K], bias float32 [N]."""
+    _on_gpu(a, weight, bias, out)
+    _check(a.dim() == 2 and a.stride(1) == 1, "linear: input must be [M, K] with unit column stride")
+    _check(weight.dim() == 2 and weight.is_contiguous(), "linear: weight must be a contiguous [N, K] matrix")
+    M, K = a.shape
+    N = weight.shape[0]
+    _check(weight.shape[1] == K, f"linear: input has K={K}, weight has K={weight.shape[1]}")
+    if bias is not None:
+        _check(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == N,
+               f"linear: bias must be float32 of {N} entries")
+    out_dtype = out_dtype or a.dtype
+    if out is None:
+        out = torch.empty(M, N, dtype=out_dtype, device=a.device)
+    _check(out.dim() == 2 and tuple(out.shape) == (M, N) and out.stride(1) == 1 and out.dtype == out_dtype,
+           "linear: bad output")
+    lda = a.stride(0) if M > 1 else K
+    ldc = out.stride(0) if M > 1 else N
+    return _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc)
+
+
+def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc) -> torch.Tensor:
+    _call("tl_gemm_generic", _ptr(a), _code(a, "linear input"), _ptr(weight), _code(weight, "linear weight"),
+          _ptr(bias), _ptr(out), _code(out, "linear output"), M, N, K, lda, ldc, _stream())
+    return out
+
+
+def rope_store(qkv: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor | None, num_heads: int,
+               num_kv_heads: int, head_dim: int, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None,
+               slots: torch.Tensor | None) -> None:
+    """Rotate the query and key heads of the fused projection ``qkv`` [T, (nq + 2 nkv) d]; queries
+    in place, rotated keys and the values into the paged cache at ``slots`` (negative: skip)."""
+    _on_gpu(qkv, pos, inv_freq, k_cache, v_cache, slots)
+    T = qkv.shape[0]
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _check(qkv.dim() == 2 and qkv.is_contiguous() and qkv.shape[1] == width,
+           f"rope_store: qkv must be contiguous [T, {width}], got {tuple(qkv.shape)}")
+    _i32(pos, "pos", T)
+    rot = 0
+    if inv_freq is not None:
+        _check(inv_freq.dtype == torch.float32 and inv_freq.is_contiguous(), "rope_store: inv_freq must be float32")
+        rot = 2 * inv_freq.numel()
+        _check(rot <= head_dim, f"rope_store: rotary width {rot} exceeds the head size {head_dim}")
+    write = k_cache is not None
+    if write:
+        _check(v_cache is not None and slots is not None, "rope_store: cache write needs k_cache, v_cache and slots")
+        for c in (k_cache, v_cache):
+            _check(c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
+                   and c.shape[2] == num_kv_heads and c.shape[3] == head_dim,
+                   "rope_store: cache must be contiguous [pages, page, nkv, d] of the activation dtype")
+        _i32(slots, "slots", T)
+    _call("tl_rope_store", _ptr(qkv), _code(qkv, "rope_store"), _ptr(pos), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache),
+          _ptr(slots), T, num_heads, num_kv_heads, head_dim, rot, 1 if write else 0, _stream())
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, tables: torch.Tensor,
+                    seq_of_token: torch.Tensor, pos: torch.Tensor, num_heads: int, num_kv_heads: int,
+                    head_dim: int, scale: float, window: int = 0, out: torch.Tensor | None = None,
+                    plan=None) -> torch.Tensor:
+    """Causal attention of each token over the cached keys of its sequence.
+
+    ``q``: [T, >= nq*d] with the query heads in the first nq*d columns (row stride free);
+    ``tables``: int32 [S, NB] page ids; ``seq_of_token``, ``pos``: int32 [T].  ``window`` > 0
+    limits a token at position p to keys [p - window + 1, p].  Returns [T, nq*d]."""
+    _on_gpu(q, k_cache, v_cache, tables, seq_of_token, pos, out)
+    T = q.shape[0]
+    _check(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= num_heads * head_dim, "paged_attention: bad query layout")
+    for c in (k_cache, v_cache):
+        _check(c.dtype == q.dtype and c.is_contiguous() and c.dim() == 4 and c.shape[2] == num_kv_heads
+               and c.shape[3] == head_dim, "paged_attention: cache must be contiguous [pages, page, nkv, d]")
+    _check(tables.dim() == 2 and tables.dtype == torch.int32 and tables.is_contiguous(), "paged_attention: bad page table")
+    _i32(seq_of_token, "seq_of_token", T)
+    _i32(pos, "pos", T)
+    if out is None:
+        out = torch.empty(T, num_heads * head_dim, dtype=q.dtype, device=q.device)
+    _check(out.dtype == q.dtype and out.dim() == 2 and out.shape[0] == T and out.stride(1) == 1, "paged_attention: bad output")
+    q_stride = q.stride(0) if T > 1 else q.shape[1]
+    o_stride = out.stride(0) if T > 1 else out.shape[1]
+    _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
+          _ptr(seq_of_token), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, num_heads,
+          num_kv_heads, head_dim, k_cache.shape[1], int(window), ctypes.c_float(scale), _stream())
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for a fused [T, 2I] projection."""
+    _on_gpu(gate_up, out)
+    _check(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0,
+           "silu_mul: input must be contiguous [T, 2I]")
+    T, I2 = gate_up.shape
+    if out is None:
+        out = torch.empty(T, I2 // 2, dtype=gate_up.dtype, device=gate_up.device)
+    _check(out.dtype == gate_up.dtype and out.is_contiguous() and tuple(out.shape) == (T, I2 // 2), "silu_mul: bad output")
+    _call("tl_silu_mul", _ptr(gate_up), _ptr(out), _code(gate_up, "silu_mul"), T, I2 // 2, _stream())
+    return out
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Row-wise arg-max of float32 logits [R, V] -> int32 [R]; the lowest index wins a tie."""
+    _on_gpu(logits, out)
+    _check(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax: logits must be float32 [R, V]")
+    R, V = logits.shape
+    if out is None:
+        out = torch.empty(R, dtype=torch.int32, device=logits.device)
+    _i32(out, "argmax output", R)
+    _call("tl_argmax", _ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(out), _stream())
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, uniform: torch.Tensor,
+           out: torch.Tensor | None = None) -> torch.Tensor:
+    """One token per row of float32 logits [R, V]: greedy where temperature <= 0, else a draw from
+    softmax(logits / temperature) cut by top-p, using the uniform number given for the row."""
+    _on_gpu(logits, temperature, top_p, uniform, out)
+    _check(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be float32 [R, V]")
+    R, V = logits.shape
+    for name, t in (("temperature", temperature), ("top_p", top_p), ("uniform", uniform)):
+        _check(t.dtype == torch.float32 and t.is_contiguous() and t.numel() == R, f"sample: {name} must be float32 [R]")
+    if out is None:
+        out = torch.empty(R, dtype=torch.int32, device=logits.device)
+    _i32(out, "sample output", R)
+    _call("tl_sample", _ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature), _ptr(top_p),
+          _ptr(uniform), _ptr(out), _stream())
+    return out

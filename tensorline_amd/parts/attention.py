@@ -1,0 +1,81 @@
+"""Grouped-query attention over the paged cache.
+
+One step: fused q/k/v projection (with bias), position encoding of queries and keys, write of the
+new keys and values into the cache, causal attention of every token of the step over the cached
+keys of its sequence, output projection (reference order: tensorline/paged.py:247-275).  All
+attention, for a whole prompt, a portion of one or a single decoded token, reads the cache; the
+step's own keys are in it before attention runs (paged.py:252-253).
+"""
+from __future__ import annotations
+
+import torch
+
+from tensorline_amd.ops import kernels
+from tensorline_amd.parts.base import Linear, Part, TensorGetter, fuse_linears
+from tensorline_amd.parts.registry import build_part, register_mixer
+from tensorline_amd.parts.spec import CacheNeed, PartSpec
+
+
+@register_mixer("attention")
+class PagedAttention(Part):
+    """Parameters: head counts and size, whether q/k/v carry a bias, the position encoding, an
+    optional ``window`` (a token sees only the last ``window`` keys, itself included), an optional
+    ``scale`` (default head_dim^-1/2, tests/test_paged_attn.py:36), and ``kv_proj`` False for a
+    layer that only reads keys and values another layer cached."""
+
+    def __init__(self, hidden_size, prefix, dtype, device, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: PartSpec, qkv_bias: bool = True, out_bias: bool = False, window: int = 0,
+                 scale: float | None = None, kv_proj: bool = True):
+        super().__init__(hidden_size, prefix, dtype, device)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
+        self.num_heads, self.num_kv_heads, self.head_dim = int(num_heads), int(num_kv_heads), int(head_dim)
+        self.window = int(window or 0)
+        self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
+        self.kv_proj = bool(kv_proj)
+        q_size, kv_size = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        self._projs = [Linear(prefix + "q_proj", hidden_size, q_size, qkv_bias)]
+        if self.kv_proj:
+            self._projs += [Linear(prefix + "k_proj", hidden_size, kv_size, qkv_bias),
+                            Linear(prefix + "v_proj", hidden_size, kv_size, qkv_bias)]
+        self.qkv: Linear | None = None
+        self.o_proj = Linear(prefix + "o_proj", q_size, hidden_size, out_bias)
+        self.position = build_part("position", position, head_dim=self.head_dim, device=device)
+
+    # ---- weights -----------------------------------------------------------------------
+    def tensors(self):
+        out = {}
+        for p in self._projs + [self.o_proj]:
+            out.update(p.tensors())
+        return out
+
+    def load(self, get: TensorGetter) -> None:
+        for p in self._projs:
+            p.load(get)
+        self.qkv = fuse_linears(self.prefix + "qkv_proj", self._projs)
+        for p in self._projs:          # the fused copy is the one that is kept
+            p.weight = p.bias = None
+        self.o_proj.load(get)
+
+    def weight_tensors(self):
+        return [t for t in (self.qkv.weight, self.qkv.bias, self.o_proj.weight, self.o_proj.bias) if t is not None]
+
+    # ---- what it keeps -------------------------------------------------------------------
+    def cache_need(self) -> CacheNeed | None:
+        return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def state_need(self):
+        return None
+
+    # ---- one step ------------------------------------------------------------------------
+    def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
+        qkv = self.qkv(h)
+        nkv_local = self.num_kv_heads if self.kv_proj else 0
+        write = cache.write and self.kv_proj
+        self.position.apply_and_store(qkv, ctx.pos, self.num_heads, nkv_local, self.head_dim,
+                                      cache.k if write else None, cache.v if write else None,
+                                      cache.slots if write else None)
+        o = kernels.paged_attention(qkv, cache.k, cache.v, cache.tables, ctx.seq_of_token, ctx.pos,
+                                    self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
+                                    window=self.window, plan=ctx.attention_plan)
+        return self.o_proj(o, out_dtype=torch.float32)

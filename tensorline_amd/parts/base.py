@@ -1,0 +1,70 @@
+"""What every part has in common: it declares the checkpoint tensors it needs and takes them.
+
+A part is built from sizes and constants only (its ``PartSpec.params``) plus ``hidden_size``,
+the checkpoint ``prefix`` it lives under, the compute ``dtype`` and the ``device``.  It does not
+know which model it is in.
+"""
+from __future__ import annotations
+
+from typing import Callable
+
+import torch
+
+from tensorline_amd.ops import kernels
+from tensorline_amd.parts.spec import TensorDecl
+
+TensorGetter = Callable[[str], torch.Tensor]
+
+
+class Part:
+    def __init__(self, hidden_size: int, prefix: str, dtype: torch.dtype, device):
+        self.hidden_size = int(hidden_size)
+        self.prefix = prefix
+        self.dtype = dtype
+        self.device = device
+
+    def tensors(self) -> dict[str, TensorDecl]:
+        """Checkpoint name -> declaration, for every tensor this part reads."""
+        return {}
+
+    def load(self, get: TensorGetter) -> None:
+        """Take the declared tensors; ``get(name)`` returns one on the device in its storage dtype."""
+
+    def weight_tensors(self) -> list[torch.Tensor]:
+        """Device tensors this part keeps (for byte accounting)."""
+        return []
+
+
+class Linear:
+    """``y = x W^T + b`` with W [out, in] as checkpoints store it (reference: tensorline/quant.py:3)."""
+
+    def __init__(self, name: str, in_features: int, out_features: int, bias: bool, std: float = 0.02):
+        self.name = name
+        self.in_features, self.out_features, self.has_bias, self.std = in_features, out_features, bias, std
+        self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
+
+    def tensors(self) -> dict[str, TensorDecl]:
+        out = {self.name + ".weight": TensorDecl((self.out_features, self.in_features), "normal", self.std, "compute")}
+        if self.has_bias:
+            out[self.name + ".bias"] = TensorDecl((self.out_features,), "normal", self.std, "float32")
+        return out
+
+    def load(self, get: TensorGetter) -> None:
+        self.weight = get(self.name + ".weight")
+        self.bias = get(self.name + ".bias") if self.has_bias else None
+
+    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+        return kernels.linear(x, self.weight, self.bias, out_dtype=out_dtype)
+
+
+def fuse_linears(name: str, parts: list[Linear]) -> Linear:
+    """One Linear whose rows are the rows of ``parts`` in order: one matrix product instead of
+    several over the same input."""
+    fused = Linear(name, parts[0].in_features, sum(p.out_features for p in parts), any(p.has_bias for p in parts))
+    fused.weight = torch.cat([p.weight for p in parts], dim=0).contiguous()
+    if fused.has_bias:
+        fused.bias = torch.cat([
+            p.bias if p.bias is not None else torch.zeros(p.out_features, dtype=torch.float32, device=p.weight.device)
+            for p in parts]).contiguous()
+    return fused

@@ -1,0 +1,47 @@
+"""Position encodings.  A position encoding owns two things: what is done to the query and key
+heads of a step's tokens given their positions, and the write of keys and values into the paged
+cache (fused, because the rotated key is what the cache holds; reference: paged.py:251-253).
+
+Interface: ``apply_and_store(qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
+slots)`` rotates the query heads of the fused projection in place and stores keys and values at
+``slots`` (``k_cache`` None: nothing is stored).
+"""
+from __future__ import annotations
+
+import torch
+
+from tensorline_amd.ops import kernels
+from tensorline_amd.parts.registry import register_position
+
+
+@register_position("rope")
+class RotaryEmbedding:
+    """Rotate-half RoPE over the first ``rotary_dim`` dims of a head:
+    theta_i = pos * base^(-2i / rotary_dim), angles in float32 (reference: fused.py:34-51; the
+    table layout cat(cos, cos) is pinned by tests/test_quant.py:116-118)."""
+
+    def __init__(self, head_dim: int, device, theta: float, rotary_dim: int | None = None):
+        self.head_dim = int(head_dim)
+        self.theta = float(theta)
+        self.rotary_dim = int(rotary_dim) if rotary_dim is not None else self.head_dim
+        if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
+            raise ValueError(f"rotary_dim {self.rotary_dim} must be even and within the head size {self.head_dim}")
+        # The exponent and the power are evaluated in float64 and rounded once to float32.
+        idx = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64)
+        inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -idx / self.rotary_dim)
+        self.inv_freq = inv.to(torch.float32).to(device)
+
+    def apply_and_store(self, qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots) -> None:
+        kernels.rope_store(qkv, pos, self.inv_freq, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots)
+
+
+@register_position("none")
+class NoPosition:
+    """No position encoding: keys and values are stored as they are."""
+
+    def __init__(self, head_dim: int, device):
+        self.head_dim = int(head_dim)
+
+    def apply_and_store(self, qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots) -> None:
+        if k_cache is not None:
+            kernels.rope_store(qkv, pos, None, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots)

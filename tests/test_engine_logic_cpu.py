@@ -1,0 +1,34 @@
+"""The engine's batch and cache logic against the plain implementation, on the CPU with kernel
+stand-ins: every way of cutting must give the plain implementation's logits."""
+import numpy as np
+import pytest
+import torch
+
+from tensorline_amd.engine.loading import load_model
+from tensorline_amd.engine.replay import TraceSession
+from tests import helpers, plain
+
+
+@pytest.fixture(scope="module", params=["A", "B", "C"])
+def setup(request, tmp_path_factory):
+    name = request.param
+    d = helpers.make_model_dir(tmp_path_factory, name, seed=3)
+    w, cfg = plain.load_folder(d)
+    lengths = {"A": [5, 17, 33, 70], "B": [1, 8, 31, 64, 100], "C": [2, 40, 65]}[name]
+    reqs = {f"r{i}": p for i, p in enumerate(helpers.prompts_for(name, lengths, seed=7))}
+    return name, d, reqs, helpers.plain_logits(w, cfg, reqs)
+
+
+@pytest.mark.parametrize("cut", ["whole", "decode", "portions", "mixed"])
+def test_cuttings_match_plain(setup, cut, cpu_kernels):
+    name, d, reqs, want = setup
+    steps = {"whole": helpers.steps_whole, "decode": helpers.steps_prefill_then_decode,
+             "portions": helpers.steps_portions, "mixed": helpers.steps_mixed}[cut](reqs)
+    model, _ = load_model(d, "float32", "cpu")
+    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=helpers.PAGE[name])
+    got = helpers.collect_logits(session.step, steps)
+    assert set(got) == set(want)
+    for key in want:
+        np.testing.assert_allclose(got[key], want[key], atol=2e-5, rtol=1e-4, err_msg=str(key))
+    assert session.cache.all_free()
+    session.cache.check()
