@@ -1,0 +1,288 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the engine's."""
+import math
+
+import pytest
+import torch
+
+from tests import plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def K():
+    from tensorline_amd.ops import kernels
+    return kernels
+
+
+def tol(dtype, f32=1e-5, bf16=2e-2):
+    return dict(atol=f32, rtol=f32) if dtype == torch.float32 else dict(atol=bf16, rtol=bf16)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(dtype):
+    torch.manual_seed(0)
+    table = torch.randn(1000, 192, device=DEV).to(dtype)
+    ids = torch.tensor([0, 999, 5, 5, 17], dtype=torch.int32, device=DEV)
+    x = K().embed(ids, table)
+    assert x.dtype == torch.float32
+    torch.testing.assert_close(x, table[ids.long()].float(), atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T", [1, 5, 64])
+def test_add_rmsnorm_reference_vector(dtype, T):
+    # sizes of the reference's own test: H=896, eps=1e-6, w ~ U(0.5, 1.5) (tests/test_quant.py:100-113)
+    torch.manual_seed(0)
+    H, eps = 896, 1e-6
+    w = torch.empty(H, device=DEV).uniform_(0.5, 1.5)
+    x = torch.randn(T, H, device=DEV)
+    r = torch.randn(T, H, device=DEV).to(dtype)
+    want_x = x + r.float()
+    want = plain.rmsnorm(want_x.double(), w.double(), eps)
+    got = K().add_rmsnorm(x, r, w, eps, dtype)
+    torch.testing.assert_close(x, want_x, atol=0, rtol=0)          # updated in place, exactly
+    torch.testing.assert_close(got.double(), want, **tol(dtype, 2e-6, 2e-2))
+    # no residual, odd width, rows picked
+    H2 = 193
+    x2 = torch.randn(7, H2, device=DEV)
+    w2 = torch.randn(H2, device=DEV)
+    keep = x2.clone()
+    got2 = K().add_rmsnorm(x2, None, w2, 1e-5, dtype)
+    torch.testing.assert_close(x2, keep, atol=0, rtol=0)
+    torch.testing.assert_close(got2.double(), plain.rmsnorm(keep.double(), w2.double(), 1e-5), **tol(dtype, 2e-6, 2e-2))
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    r2 = torch.randn(7, H2, device=DEV).to(dtype)
+    got3 = K().add_rmsnorm(x2, r2, w2, 1e-5, dtype, rows=rows)
+    torch.testing.assert_close(x2, keep, atol=0, rtol=0)            # with rows, x is left alone
+    want3 = plain.rmsnorm((keep + r2.float())[rows.long()].double(), w2.double(), 1e-5)
+    torch.testing.assert_close(got3.double(), want3, **tol(dtype, 2e-6, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 64, 130])
+@pytest.mark.parametrize("N,Kd", [(176, 64), (1000, 192), (64, 100), (3, 7)])
+def test_linear(dtype, M, N, Kd):
+    torch.manual_seed(M * 1000 + N)
+    a = torch.randn(M, Kd, device=DEV).to(dtype)
+    w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(dtype)
+    b = torch.randn(N, device=DEV)
+    want = a.double() @ w.double().T + b.double()
+    got = K().linear(a, w, b)
+    assert got.dtype == dtype
+    torch.testing.assert_close(got.double(), want, **tol(dtype, 1e-5, 3e-2))
+    got32 = K().linear(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(got32.double(), a.double() @ w.double().T, **tol(dtype, 1e-5, 1e-5))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear_strided_rows(dtype):
+    torch.manual_seed(1)
+    big = torch.randn(9, 300, device=DEV).to(dtype)
+    a = big[:, 20:120]
+    w = torch.randn(33, 100, device=DEV).to(dtype)
+    got = K().linear(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(got.double(), a.double() @ w.double().T, **tol(dtype, 2e-5, 2e-5))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,rot", [(14, 2, 64, 64), (5, 1, 48, 48), (4, 4, 16, 8), (28, 4, 128, 128)])
+def test_rope_store(dtype, nq, nkv, d, rot):
+    torch.manual_seed(0)
+    T, bs, pages, theta = 37, 8, 12, 50000.0
+    qkv = torch.randn(T, (nq + 2 * nkv) * d, device=DEV).to(dtype)
+    pos = torch.randint(0, 3000, (T,), dtype=torch.int32, device=DEV)
+    slots = torch.randperm(pages * bs, device=DEV)[:T].to(torch.int32)
+    slots[5] = -1
+    kc = torch.full((pages, bs, nkv, d), 7.0, device=DEV).to(dtype)
+    vc = torch.full((pages, bs, nkv, d), 7.0, device=DEV).to(dtype)
+    i = torch.arange(0, rot, 2, dtype=torch.float64)
+    inv_freq = (theta ** (-i / rot)).float().to(DEV)
+    heads = qkv.float().cpu().view(T, nq + 2 * nkv, d)
+    want_q = plain.rope(heads[:, :nq], pos.cpu(), theta, rot)
+    want_k = plain.rope(heads[:, nq:nq + nkv], pos.cpu(), theta, rot)
+    want_v = heads[:, nq + nkv:]
+    K().rope_store(qkv, pos, inv_freq, nq, nkv, d, kc, vc, slots)
+    got = qkv.float().cpu().view(T, nq + 2 * nkv, d)
+    t = tol(dtype, 2e-5, 2e-2)
+    torch.testing.assert_close(got[:, :nq], want_q, **t)
+    kf, vf = kc.float().cpu().view(-1, nkv, d), vc.float().cpu().view(-1, nkv, d)
+    ok = slots.cpu() >= 0
+    torch.testing.assert_close(kf[slots.cpu()[ok].long()], want_k[ok], **t)
+    torch.testing.assert_close(vf[slots.cpu()[ok].long()], want_v[ok], atol=0, rtol=0)
+    untouched = torch.ones(pages * bs, dtype=torch.bool)
+    untouched[slots.cpu()[ok].long()] = False
+    assert torch.all(kf[untouched] == 7.0) and torch.all(vf[untouched] == 7.0)
+    # position 0 is the identity
+    qkv0 = torch.randn(3, (nq + 2 * nkv) * d, device=DEV).to(dtype)
+    keep = qkv0.clone()
+    K().rope_store(qkv0, torch.zeros(3, dtype=torch.int32, device=DEV), inv_freq, nq, nkv, d, None, None, None)
+    torch.testing.assert_close(qkv0, keep, atol=0, rtol=0)
+
+
+def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False):
+    """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries."""
+    torch.manual_seed(seed)
+    S = len(lens)
+    q_lens = q_lens or [1] * S
+    nb = max(-(-n // bs) for n in lens)
+    num_blocks = S * nb + 8
+    kc = torch.randn(num_blocks, bs, nkv, d, device=DEV).to(dtype)
+    vc = torch.randn(num_blocks, bs, nkv, d, device=DEV).to(dtype)
+    tables = torch.randperm(num_blocks, device=DEV)[:S * nb].view(S, nb).to(torch.int32)   # scattered pages
+    seq_of, pos = [], []
+    for s, (n, ql) in enumerate(zip(lens, q_lens)):
+        for p in range(n - ql, n):
+            seq_of.append(s)
+            pos.append(p)
+    T = len(pos)
+    q = torch.randn(T, nq * d, device=DEV).to(dtype)
+    if spike:
+        # one far key among hundreds must dominate: scale a query and a matching early key
+        kflat = kc.view(-1, nkv, d)
+        for t in range(T):
+            s = seq_of[t]
+            far = 1 if lens[s] > 2 else 0
+            row = int(tables[s, far // bs]) * bs + far % bs
+            kflat[row] = (q[t].view(nq, d)[:nkv].float() * 4).to(dtype)
+    out = K().paged_attention(q, kc, vc, tables, torch.tensor(seq_of, dtype=torch.int32, device=DEV),
+                              torch.tensor(pos, dtype=torch.int32, device=DEV), nq, nkv, d, d ** -0.5, window=window)
+    kf, vf = kc.double().cpu().view(-1, nkv, d), vc.double().cpu().view(-1, nkv, d)
+    want = torch.empty(T, nq, d, dtype=torch.float64)
+    tcpu = tables.cpu().long()
+    t0 = 0
+    for s, (n, ql) in enumerate(zip(lens, q_lens)):
+        keys = torch.arange(n)
+        rows = tcpu[s][keys // bs] * bs + keys % bs
+        qs = q[t0:t0 + ql].double().cpu().view(ql, nq, d)
+        want[t0:t0 + ql] = plain.causal_attention(qs, kf[rows], vf[rows], d ** -0.5, window=window, q_offset=n - ql)
+        t0 += ql
+    return out.double().cpu().view(T, nq, d), want
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads", [(14, 2), (12, 2), (16, 2), (4, 4)])
+@pytest.mark.parametrize("lens", [[1], [15, 16, 17], [63, 64, 65, 300], [1400] * 3 + [2, 129]])
+def test_attention_decode_reference_cases(dtype, heads, lens):
+    # the cases of the reference's kernel test (tests/test_paged_attn.py:22-38): D=64, page 16
+    got, want = _attention_case(dtype, heads[0], heads[1], 64, 16, lens)
+    torch.testing.assert_close(got, want, **tol(dtype, 2e-5, 1e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,bs", [(5, 1, 48, 16), (4, 2, 16, 8), (28, 4, 128, 16), (6, 2, 32, 8), (3, 3, 80, 4)])
+def test_attention_portions_and_spike(dtype, nq, nkv, d, bs):
+    lens, q_lens = [70, 9, 300, 2], [33, 9, 2, 1]
+    got, want = _attention_case(dtype, nq, nkv, d, bs, lens, q_lens, spike=True, seed=3)
+    torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 7, 16, 100])
+def test_attention_window(dtype, window):
+    got, want = _attention_case(dtype, 6, 2, 32, 8, [50, 7, 130], [20, 7, 1], window=window, seed=5)
+    torch.testing.assert_close(got, want, **tol(dtype, 2e-5, 1e-2))
+
+
+def test_attention_special_cases():
+    # one key: o = v;  q = 0: o = mean of the visible values
+    dtype, nq, nkv, d, bs = torch.float32, 4, 2, 16, 8
+    kc = torch.randn(4, bs, nkv, d, device=DEV)
+    vc = torch.randn(4, bs, nkv, d, device=DEV)
+    tables = torch.tensor([[2, 0]], dtype=torch.int32, device=DEV)
+    z = torch.zeros(1, dtype=torch.int32, device=DEV)
+    q = torch.randn(1, nq * d, device=DEV)
+    o = K().paged_attention(q, kc, vc, tables, z, z, nq, nkv, d, 0.25).view(nq, d)
+    torch.testing.assert_close(o, vc[2, 0].repeat_interleave(2, 0), atol=1e-6, rtol=1e-6)
+    p = torch.tensor([10], dtype=torch.int32, device=DEV)
+    o = K().paged_attention(torch.zeros_like(q), kc, vc, tables, z, p, nq, nkv, d, 0.25).view(nq, d)
+    vis = torch.cat([vc[2], vc[0, :3]]).mean(0)
+    torch.testing.assert_close(o, vis.repeat_interleave(2, 0), atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    torch.manual_seed(0)
+    gu = (torch.randn(9, 2 * 176, device=DEV) * 3).to(dtype)
+    got = K().silu_mul(gu)
+    g, u = gu[:, :176].double(), gu[:, 176:].double()
+    torch.testing.assert_close(got.double(), torch.nn.functional.silu(g) * u, **tol(dtype, 1e-5, 2e-2))
+
+
+def test_argmax_and_ties():
+    torch.manual_seed(0)
+    lg = torch.randn(6, 1000, device=DEV)
+    lg[2, 17] = lg[2, 900] = 50.0        # tie: the lower index wins
+    got = K().argmax(lg)
+    want = lg.argmax(-1)
+    want[2] = 17
+    assert got.tolist() == want.tolist()
+    big = torch.randn(3, 152064, device=DEV)
+    assert K().argmax(big).tolist() == big.argmax(-1).tolist()
+
+
+def test_sample_keep_rule_and_draws():
+    # hand vector of the keep rule: p = [.5, .3, .2]; top_p .5 keeps one token, .51 keeps two
+    lg = torch.log(torch.tensor([[0.5, 0.3, 0.2]], device=DEV))
+    one = torch.ones(1, device=DEV)
+    for tp, u, want in [(0.5, 0.99, 0), (0.51, 0.99, 1), (0.51, 0.1, 0), (0.81, 0.99, 2), (1.0, 0.99, 2), (1.0, 0.6, 1)]:
+        got = K().sample(lg, one, one * tp, one * u)
+        assert got.tolist() == [want], (tp, u, got.tolist())
+    # greedy rows inside a sampling batch, and agreement with the plain rule on random rows
+    torch.manual_seed(1)
+    R, V = 64, 1000
+    lg = torch.randn(R, V, device=DEV) * 3
+    temp = torch.rand(R, device=DEV) + 0.3
+    temp[::7] = 0.0
+    tp = torch.rand(R, device=DEV) * 0.9 + 0.1
+    tp[::5] = 1.0
+    u = torch.rand(R, device=DEV)
+    got = K().sample(lg, temp, tp, u).tolist()
+    miss = 0
+    for r in range(R):
+        want = plain.sample_with_uniform(lg[r].cpu(), float(temp[r]), float(tp[r]), float(u[r]))
+        if temp[r] <= 0:
+            assert got[r] == want
+        elif got[r] != want:
+            # a float32 running sum may land on the other side of a boundary next to the target
+            probs = torch.softmax(lg[r].double().cpu() / float(temp[r]), -1)
+            if tp[r] < 1:
+                assert plain.top_p_keep(probs, float(tp[r]))[got[r]], "drew a token outside the kept set"
+            miss += 1
+    assert miss <= 2
+    # same inputs, same tokens, whatever else is in the batch
+    again = K().sample(lg[10:20].contiguous(), temp[10:20].contiguous(), tp[10:20].contiguous(), u[10:20].contiguous())
+    assert again.tolist() == got[10:20]
+
+
+def test_sample_frequencies():
+    torch.manual_seed(2)
+    V, R = 50, 20000
+    row = torch.randn(V, device=DEV) * 2
+    lg = row.repeat(R, 1)
+    u = torch.rand(R, device=DEV)
+    t = torch.full((R,), 0.8, device=DEV)
+    got = K().sample(lg, t, torch.ones(R, device=DEV), u)
+    freq = torch.bincount(got.long(), minlength=V).double().cpu() / R
+    probs = torch.softmax(row.double().cpu() / 0.8, -1)
+    assert (freq - probs).abs().max() < 0.015
+    # temperature -> 0+ is arg-max
+    cold = K().sample(lg[:4], torch.full((4,), 1e-4, device=DEV), torch.ones(4, device=DEV), u[:4])
+    assert cold.tolist() == [int(row.argmax())] * 4
+
+
+def test_bad_arguments_are_refused():
+    from tensorline_amd.ops.kernels import KernelError
+    with pytest.raises(KernelError):
+        K().linear(torch.randn(2, 8, device=DEV), torch.randn(4, 9, device=DEV))
+    with pytest.raises(KernelError):
+        K().embed(torch.zeros(2, dtype=torch.int64, device=DEV), torch.randn(4, 8, device=DEV))
+    with pytest.raises(KernelError):
+        K().add_rmsnorm(torch.randn(2, 8), None, torch.ones(8), 1e-6, torch.float32)
+    with pytest.raises(KernelError):
+        kc = torch.randn(2, 4, 1, 512, device=DEV)
+        K().paged_attention(torch.randn(1, 512, device=DEV), kc, kc, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                            torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
+                            1, 1, 512, 1.0)
