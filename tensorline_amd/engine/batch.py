@@ -152,6 +152,7 @@ def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[
         pos[r0] = 0
         seq_of[r0] = s
         q_start[s] = r0
+        rows.append(r0)           # a fixed-shape batch has a logits row for every sequence
         r0 += 1
     q_start[S_pad] = r0
 
