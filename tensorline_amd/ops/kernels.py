@@ -153,6 +153,8 @@ def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
                f"linear: bias must be float32 of {N} entries")
     out_dtype = out_dtype or a.dtype
     if out is None:
+        if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M > SKINNY_MAX_ROWS:
+            return _library_linear(a, weight, bias, out_dtype)
         out = torch.empty(M, N, dtype=out_dtype, device=a.device)
     _check(out.dim() == 2 and tuple(out.shape) == (M, N) and out.stride(1) == 1 and out.dtype == out_dtype,
            "linear: bad output")
@@ -161,10 +163,65 @@ def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     return _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc)
 
 
+SKINNY_MAX_ROWS = 64
+
+
+def _skinny_ok(a: torch.Tensor, weight: torch.Tensor, M: int, K: int, lda: int) -> bool:
+    return (a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS
+            and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
 def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc) -> torch.Tensor:
+    """bfloat16 with few rows: the streaming MFMA kernel.  float32, and shapes that kernel does not
+    take: the plain tiled kernel.  (bfloat16 with many rows went to the library before this, where
+    the reference uses one too: tensorline/paged.py:179-188.)"""
+    if _skinny_ok(a, weight, M, K, lda):
+        _call("tl_gemm_skinny", _ptr(a), _ptr(weight), _ptr(bias), _ptr(out), _code(out, "linear output"),
+              M, N, K, lda, ldc, _stream())
+        return out
     _call("tl_gemm_generic", _ptr(a), _code(a, "linear input"), _ptr(weight), _code(weight, "linear weight"),
           _ptr(bias), _ptr(out), _code(out, "linear output"), M, N, K, lda, ldc, _stream())
     return out
+
+
+_MM_OUT_DTYPE_OK: bool | None = None
+
+
+def _library_linear(a, weight, bias, out_dtype) -> torch.Tensor:
+    """hipBLASLt through torch for many-row bfloat16 products (float32 accumulation inside)."""
+    global _MM_OUT_DTYPE_OK
+    wt = weight.t()
+    if out_dtype == torch.float32:
+        if _MM_OUT_DTYPE_OK is None:
+            try:
+                torch.mm(a[:1], wt[:, :16], out_dtype=torch.float32)
+                _MM_OUT_DTYPE_OK = True
+            except Exception:
+                _MM_OUT_DTYPE_OK = False
+        y = torch.mm(a, wt, out_dtype=torch.float32) if _MM_OUT_DTYPE_OK else torch.mm(a, wt).to(torch.float32)
+        if bias is not None:
+            y.add_(bias)
+        return y
+    y = torch.mm(a, wt)
+    if bias is not None:
+        y.add_(bias.to(y.dtype))
+    return y
+
+
+def swiglu_gate_up(h: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+    """``silu(h Wg^T) * (h Wu^T)`` for a fused [2I, K] weight (gate rows first): one kernel for
+    few-row bfloat16 batches, product then SiLU-multiply otherwise."""
+    _on_gpu(h, gate_up_weight)
+    _check(h.dim() == 2 and h.stride(1) == 1 and gate_up_weight.dim() == 2 and gate_up_weight.is_contiguous()
+           and gate_up_weight.shape[0] % 2 == 0 and gate_up_weight.shape[1] == h.shape[1], "swiglu_gate_up: bad shapes")
+    M, K = h.shape
+    I = gate_up_weight.shape[0] // 2
+    lda = h.stride(0) if M > 1 else K
+    if _skinny_ok(h, gate_up_weight, M, K, lda):
+        out = torch.empty(M, I, dtype=h.dtype, device=h.device)
+        _call("tl_gemm_skinny_swiglu", _ptr(h), _ptr(gate_up_weight), _ptr(out), M, I, K, lda, I, _stream())
+        return out
+    return silu_mul(linear(h, gate_up_weight))
 
 
 def rope_store(qkv: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor | None, num_heads: int,

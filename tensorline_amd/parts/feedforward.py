@@ -37,5 +37,5 @@ class SwiGLU(Part):
         return [self.gate_up.weight, self.down.weight]
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
-        act = kernels.silu_mul(self.gate_up(h))
+        act = kernels.swiglu_gate_up(h, self.gate_up.weight)
         return self.down(act, out_dtype=torch.float32)

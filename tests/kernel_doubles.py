@@ -86,6 +86,10 @@ def silu_mul(gate_up, out=None):
     return (g * torch.sigmoid(g) * u).to(gate_up.dtype)
 
 
+def swiglu_gate_up(h, gate_up_weight):
+    return silu_mul(linear(h, gate_up_weight))
+
+
 def argmax(logits, out=None):
     return logits.argmax(-1).to(torch.int32)
 
@@ -110,7 +114,7 @@ def sample(logits, temperature, top_p, uniform, out=None):
     return res
 
 
-ALL = ["require_gpu", "embed", "add_rmsnorm", "linear", "rope_store", "paged_attention", "silu_mul", "argmax",
+ALL = ["require_gpu", "embed", "add_rmsnorm", "linear", "rope_store", "paged_attention", "silu_mul", "swiglu_gate_up", "argmax",
        "sample"]
 
 

@@ -77,6 +77,39 @@ def test_linear(dtype, M, N, Kd):
     torch.testing.assert_close(got32.double(), a.double() @ w.double().T, **tol(dtype, 1e-5, 1e-5))
 
 
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("N,Kd", [(1000, 1184), (4608, 3584), (136, 8), (50, 264)])
+def test_linear_few_rows_bfloat16(M, N, Kd):
+    """The streaming MFMA kernel: every M up to 64, N no multiple of 16, K with a partial chunk."""
+    torch.manual_seed(M + N)
+    a = torch.randn(M, Kd, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(torch.bfloat16)
+    b = torch.randn(N, device=DEV)
+    want = a.double() @ w.double().T + b.double()
+    got = K().linear(a, w, b, out_dtype=torch.float32)
+    torch.testing.assert_close(got.double(), want, atol=2e-4, rtol=2e-4)
+    got16 = K().linear(a, w, b)
+    torch.testing.assert_close(got16.double(), want, atol=3e-2, rtol=3e-2)
+    # the value of a row does not depend on the rows beside it
+    alone = K().linear(a[M - 1:M].contiguous(), w, b, out_dtype=torch.float32)
+    torch.testing.assert_close(alone[0], got[M - 1], atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M", [1, 8, 40, 64, 200])
+@pytest.mark.parametrize("I,Kd", [(176, 64), (1184, 3584), (100, 48)])
+def test_swiglu_gate_up(dtype, M, I, Kd):
+    torch.manual_seed(M + I)
+    h = torch.randn(M, Kd, device=DEV).to(dtype)
+    w = (torch.randn(2 * I, Kd, device=DEV) / math.sqrt(Kd) * 2).to(dtype)
+    got = K().swiglu_gate_up(h, w)
+    gu = h.double() @ w.double().T
+    want = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+    assert got.dtype == dtype and tuple(got.shape) == (M, I)
+    # float32 accumulation over K terms: the error grows with sqrt(K)
+    torch.testing.assert_close(got.double(), want, **tol(dtype, 2e-6 * math.sqrt(Kd) + 1e-5, 4e-2))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_linear_strided_rows(dtype):
     torch.manual_seed(1)
