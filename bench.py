@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at the Qwen2.5-7B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
+
+A step is one decode step of the whole batch through the engine loop (schedule, one graph replay
+of the model, sampling, accept).  Weights are random (generated on the GPU from a seed), prompts
+are token ids uniform over the vocabulary.  One JSON line is printed: decoded tokens per second
+at the default batch, the prefill of one 2,048-token prompt, the decode step's share of the HBM
+roofline, and decode throughput at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_GBPS = 8000.0
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+# layer sizes of the Qwen2.5-7B shape
+SHAPE_7B = dict(vocab_size=152064, hidden_size=3584, intermediate_size=18944, num_hidden_layers=28,
+                num_attention_heads=28, num_key_value_heads=4, head_dim=128, rope_theta=1000000.0,
+                rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768)
+
+
+def make_config(layers: int | None):
+    from tensorline_amd.config import Qwen2Config
+    d = dict(SHAPE_7B, architectures=["Qwen2ForCausalLM"])
+    if layers:
+        d["num_hidden_layers"] = layers
+    return Qwen2Config.from_dict(d)
+
+
+def layer_matrix_params(cfg) -> int:
+    H, I = cfg.hidden_size, cfg.intermediate_size
+    return (cfg.q_size + 2 * cfg.kv_size) * H + cfg.q_size * H + 3 * H * I
+
+
+def decode_bytes(cfg, batch: int, context: int, elem: int = 2) -> float:
+    """Bytes a decode step has to read: every weight it uses once, and the cache of the live requests."""
+    L, H, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.vocab_size
+    weights = (L * layer_matrix_params(cfg) + V * H) * elem
+    weights += L * (cfg.q_size + 2 * cfg.kv_size) * 4 + (2 * L + 1) * H * 4          # biases and norm weights
+    weights += batch * H * elem                                                        # embedding rows
+    kv = batch * context * 2 * cfg.kv_size * elem * L
+    return float(weights + kv)
+
+
+def prefill_flops(cfg, tokens: int, rows: int = 1) -> float:
+    L, V, H = cfg.num_hidden_layers, cfg.vocab_size, cfg.hidden_size
+    linear = 2.0 * tokens * L * layer_matrix_params(cfg)
+    attn = 4.0 * cfg.num_attention_heads * cfg.head_dim * (tokens * (tokens + 1) / 2) * L
+    head = 2.0 * rows * V * H
+    return linear + attn + head
+
+
+def random_prompts(n: int, length: int, vocab: int, seed: int):
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, vocab, size=length).tolist() for _ in range(n)]
+
+
+def sync():
+    import torch
+    torch.cuda.synchronize()
+
+
+def bench_decode(llm, batch: int, context: int, steps: int, warmup: int, seed: int) -> dict:
+    """Fill ``batch`` sequences so that the last timed step runs at ``context`` tokens, then time
+    ``steps`` decode steps of the whole batch."""
+    from tensorline_amd import SamplingParams
+    cfg = llm.model_config
+    prompt_len = context - (warmup + steps)
+    assert prompt_len >= 1
+    eng = llm.engine
+    reqs = [eng.add_request(p, SamplingParams(max_tokens=warmup + steps + 8, stop_token_ids={-1}))
+            for p in random_prompts(batch, prompt_len, cfg.vocab_size, seed)]
+    t0 = time.perf_counter()
+    while any(r.num_computed < r.prompt_len for r in reqs):          # prefill, in portions
+        eng.step()
+    sync()
+    fill_s = time.perf_counter() - t0
+    for _ in range(warmup):
+        eng.step()
+    sync()
+    replays0 = eng.counters()["graph_replays"]
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        eng.step()
+    sync()
+    dt = time.perf_counter() - t0
+    assert all(r.num_generated >= warmup + steps for r in reqs), "a decode step did not advance every sequence"
+    out = {"tok_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3, "fill_s": fill_s,
+           "graph_replays": eng.counters()["graph_replays"] - replays0}
+    for r in reqs:
+        eng.abort(r)
+    assert llm.cache.all_free()
+    return out
+
+
+def bench_prefill(llm, tokens: int, reps: int, seed: int) -> dict:
+    """One prompt of ``tokens`` tokens in one step, logits for its last position."""
+    from tensorline_amd.engine.batch import StepEntry
+    cfg = llm.model_config
+    cache, runner = llm.cache, llm.engine.runner
+    prompt = random_prompts(1, tokens, cfg.vocab_size, seed)[0]
+    times = []
+    for i in range(reps + 1):
+        rid = ("prefill", i)
+        cache.add_request(rid)
+        assert cache.grow(rid, tokens)
+        sync()
+        t0 = time.perf_counter()
+        logits = runner.step([StepEntry(rid, prompt, 0, [tokens - 1])])
+        logits.argmax(-1).tolist()
+        sync()
+        times.append(time.perf_counter() - t0)
+        cache.release(rid)
+    best = min(times[1:])                                              # the first run warms up
+    return {"s": best, "tok_s": tokens / best}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
+    ap.add_argument("--dtype", default="bfloat16")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
+    ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    from tensorline_amd import LLM
+    cfg = make_config(args.layers)
+    full_layers = SHAPE_7B["num_hidden_layers"]
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    max_len = args.context + 16
+    page = 16
+    llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
+              num_blocks=max_batch * (-(-max_len // page)) + 8, max_num_seqs=max_batch, max_batched_tokens=2048,
+              max_model_len=max_len, graphs=not args.no_graphs, graph_warmup_tokens=0, prefix_caching=False)
+    elem = 2 if args.dtype in ("bfloat16", "bf16") else 4
+    dtype_key = "bfloat16" if elem == 2 else "float32"
+
+    main_run = bench_decode(llm, args.batch, args.context, args.steps, args.warmup, args.seed + 1)
+    pre = bench_prefill(llm, args.prefill_tokens, 3, args.seed + 2)
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            k = max(8, args.steps // 2)
+            points[f"decode_b{b}"] = round(bench_decode(llm, b, args.context, k, 4, args.seed + 3 + b)["tok_s"], 1)
+
+    step_s = main_run["ms_per_step"] / 1e3
+    mean_ctx = args.context - args.steps / 2.0
+    achieved = decode_bytes(cfg, args.batch, int(mean_ctx), elem) / step_s / 1e9
+    flops = prefill_flops(cfg, args.prefill_tokens)
+    line = {
+        "metric": "decode tok/s @ batch 8, context 4096 (Qwen2.5-7B shape)",
+        "value": round(main_run["tok_s"], 1),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_run["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if elem == 2 else "fp32",
+        "data": "synthetic: random weights from a seed, token ids uniform over the vocabulary",
+        "config": {
+            "model": "Qwen2.5-7B shape", "global_batch": args.batch, "seq_len": args.context,
+            "parallelism": "single GPU", "layers": cfg.num_hidden_layers, "layers_of_shape": full_layers,
+            "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
+            "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "page_size": page,
+            "prefill_tokens": args.prefill_tokens, "graphs": not args.no_graphs, "sampling": "greedy",
+            "decode_graph_replays": main_run["graph_replays"],
+        },
+        "prefill": {"value": round(pre["tok_s"], 1), "tokens": args.prefill_tokens, "ms": round(pre["s"] * 1e3, 3),
+                    "frac": round(flops / pre["s"] / PEAK_FLOPS[dtype_key], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBPS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    torch.cuda.synchronize()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -109,10 +109,12 @@ class CacheManager:
 
         if allocate_storage:
             for g in self.groups:
-                shape = (num_blocks + 1, page_size, g.need.num_kv_heads, g.need.head_dim)
+                # keys [pages, page, nkv, d]; values transposed within the page: [pages, nkv, d, page]
+                k_shape = (num_blocks + 1, page_size, g.need.num_kv_heads, g.need.head_dim)
+                v_shape = (num_blocks + 1, g.need.num_kv_heads, g.need.head_dim, page_size)
                 for i in g.entries:
-                    g.k[i] = torch.zeros(shape, dtype=dtype, device=device)
-                    g.v[i] = torch.zeros(shape, dtype=dtype, device=device)
+                    g.k[i] = torch.zeros(k_shape, dtype=dtype, device=device)
+                    g.v[i] = torch.zeros(v_shape, dtype=dtype, device=device)
             for i, need in enumerate(self.state_needs):
                 if need is not None:
                     self.state[i] = torch.zeros((max_requests + 1, *need.shape), dtype=_TORCH_DTYPES[need.dtype], device=device)

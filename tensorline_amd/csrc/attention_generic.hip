@@ -4,7 +4,8 @@
 //
 // A token at position p of sequence s attends to keys [lo, p] of that sequence, lo = 0 or
 // p - window + 1 for a windowed layer, found through the sequence's row of the page table.  The
-// keys of the step's own tokens are already in the cache when this runs.  Scores, the running
+// keys of the step's own tokens are already in the cache when this runs.  k_cache is
+// [pages, page, nkv, d]; v_cache is [pages, nkv, d, page].  Scores, the running
 // maximum, the sum and the accumulator are float (reference: tensorline/paged_attn.py:25-58,
 // tensorline/paged.py:233-238).  Key tiles start at lo, so the result for a position does not
 // depend on how the sequence was cut into steps.
@@ -93,7 +94,8 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
             const int nkeys = (hi - k0 < AG_TILE) ? hi - k0 : AG_TILE;
             if (c < d) {
                 for (int j = sub; j < nkeys; j += nsub) {
-                    const float vv = tl_to_float(v_cache[((size_t)blk_s[j] * nkv + kvh) * d + c]);
+                    const int vrow = blk_s[j];
+                    const float vv = tl_to_float(v_cache[(((size_t)(vrow / bs) * nkv + kvh) * d + c) * bs + vrow % bs]);
 #pragma unroll
                     for (int g = 0; g < AG_GC; ++g)
                         if (g < gc) acc[g] = fmaf(s_s[g * AG_TILE + j], vv, acc[g]);

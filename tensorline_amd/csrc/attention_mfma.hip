@@ -1,0 +1,295 @@
+// Causal grouped-query attention over the paged cache on the matrix cores (bfloat16, gfx950),
+// for prompt portions and decoded tokens alike, with the key range optionally split over several
+// waves (split-KV) and a second kernel that merges the splits.
+//
+// Work of one wave: NT tiles of 16 "columns" of one (sequence, key/value head).  A column is a
+// (query token, query head of the group) pair; columns are numbered token-major, so a decoded
+// token with a group of 7 fills 7 of the 16 columns of one tile and a prompt portion fills whole
+// tiles.  The wave walks its share of the keys in blocks of 32 and keeps, per column, the running
+// maximum, the running sum and the output accumulator in float (online softmax; reference:
+// tensorline/paged_attn.py:25-58).  Waves never talk to each other: no LDS, no barriers.
+//
+// Matrix-core mapping (v_mfma_f32_16x16x32_bf16, D = A*B, lane l: c = l % 16, g = l / 16):
+//   scores^T [keys x columns] = K [keys x d] * Q^T [d x columns]
+//       A = K: lane holds 8 dims of key row c;  B = Q^T: lane holds the same 8 dims of column c.
+//       The accumulator register i of lane l is (key row 4g + i, column c).
+//   out^T [d x columns] += V^T [d x keys] * P^T [keys x columns]
+//       A = V^T: lane holds 8 keys of dim c;     B = P^T: lane holds the same 8 keys of column c.
+// Which key a key row stands for is free.  The two score tiles of a 32-key block use rows
+//   tile 0: row 4g + i  <->  key 8g + i          tile 1: row 4g + i  <->  key 8g + 4 + i
+// so that after both tiles lane (c, g) holds exactly the probabilities of keys 8g .. 8g+7 of
+// column c: the B fragment of the second product, with no exchange between lanes.  The matching A
+// fragment, 8 consecutive keys of one dim, is one 16-byte load because the value cache is stored
+// transposed within a page: [pages, nkv, d, page].  The key cache is [pages, page, nkv, d].
+//
+// Key blocks are aligned to absolute positions (block b holds keys 32b .. 32b+31), and so are the
+// splits (split s holds blocks s*SB .. s*SB + SB - 1): which keys are summed together does not
+// depend on the context length, on the launch's number of splits or on how the sequence was cut
+// into steps.  A wave whose split holds none of its keys writes nothing; the merge kernel visits
+// exactly the splits that hold keys of a token.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8 am_frag(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+__device__ __forceinline__ uint32_t am_pack2(float a, float b) {
+    return (uint32_t)tl_f2bf_bits(a) | ((uint32_t)tl_f2bf_bits(b) << 16);
+}
+
+template <int DC, int NT>
+__global__ __launch_bounds__(256) void attn_mfma_kernel(
+    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+    const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, float* __restrict__ ws_o,
+    float* __restrict__ ws_ml, int nq, int nkv, int bs, int window, float scale, int nsplit, int split_blocks) {
+    constexpr int D = DC * 32;
+    constexpr int DB = D / 16;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int s = blockIdx.x, kvh = blockIdx.y;
+    const int widx = blockIdx.z * 4 + wave;
+    const int tg = widx / nsplit, sp = widx - tg * nsplit;
+    const int G = nq / nkv;
+    const int r0 = q_start[s];
+    const int n = q_start[s + 1] - r0;
+    const int start = ctx_start[s];
+    const int ncols = n * G;
+    const int col0 = tg * NT * 16;
+    if (col0 >= ncols) return;
+    const int32_t* table = tables + (size_t)s * NB;
+
+    // ---- this lane's column of each tile ----
+    uint4 qf[NT][DC];
+    int p_col[NT], lo_col[NT], row_col[NT], head_col[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int col = col0 + j * 16 + c;
+        const bool valid = col < ncols;
+        const int tok = valid ? col / G : 0;
+        const int gh = valid ? col - tok * G : 0;
+        row_col[j] = r0 + tok;
+        head_col[j] = kvh * G + gh;
+        p_col[j] = valid ? start + tok : -1;                  // -1: every key is masked
+        lo_col[j] = (window > 0 && p_col[j] - window + 1 > 0) ? p_col[j] - window + 1 : 0;
+        const bf16_t* qp = q + (size_t)row_col[j] * q_stride + (size_t)head_col[j] * D + g * 8;
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc)
+            qf[j][dc] = valid ? *reinterpret_cast<const uint4*>(qp + dc * 32) : make_uint4(0, 0, 0, 0);
+    }
+
+    // ---- key range of the wave, in blocks of 32, and this split's share ----
+    const int last_col = ((col0 + NT * 16 < ncols) ? col0 + NT * 16 : ncols) - 1;
+    const int khi = start + last_col / G;                      // last key any column of the wave sees
+    int klo = 0;
+    if (window > 0) {
+        klo = start + col0 / G - window + 1;
+        if (klo < 0) klo = 0;
+    }
+    const int b_lo = klo >> 5, b_hi = khi >> 5;
+    int bb = b_lo, be = b_hi + 1;
+    if (nsplit > 1) {
+        if (sp * split_blocks > bb) bb = sp * split_blocks;
+        if ((sp + 1) * split_blocks < be) be = (sp + 1) * split_blocks;
+        if (bb >= be) return;
+    }
+
+    float m_run[NT], l_run[NT];
+    f32x4 acc[NT][DB];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        m_run[j] = -INFINITY;
+        l_run[j] = 0.f;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) acc[j][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int krow_in_block0 = 8 * (c >> 2) + (c & 3);         // key of row c in tile 0; tile 1: + 4
+    for (int b = bb; b < be; ++b) {
+        const int kb = b << 5;
+        // keys past khi are masked for every column; their addresses are clamped to stay on
+        // pages the sequence owns
+        int k0 = kb + krow_in_block0, k1 = k0 + 4;
+        if (k0 > khi) k0 = khi;
+        if (k1 > khi) k1 = khi;
+        const bf16_t* kp0 = kc + ((size_t)(table[k0 / bs] * bs + k0 % bs) * nkv + kvh) * D + g * 8;
+        const bf16_t* kp1 = kc + ((size_t)(table[k1 / bs] * bs + k1 % bs) * nkv + kvh) * D + g * 8;
+        uint4 kf0[DC], kf1[DC];
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+            kf0[dc] = *reinterpret_cast<const uint4*>(kp0 + dc * 32);
+            kf1[dc] = *reinterpret_cast<const uint4*>(kp1 + dc * 32);
+        }
+        int vk = kb + 8 * g;
+        if (vk > khi) vk = khi & ~7;
+        const bf16_t* vp = vc + (((size_t)table[vk / bs] * nkv + kvh) * D + c) * bs + vk % bs;
+        uint4 vf[DB];
+#pragma unroll
+        for (int db = 0; db < DB; ++db) vf[db] = *reinterpret_cast<const uint4*>(vp + (size_t)db * 16 * bs);
+
+        const int key_base = kb + 8 * g;                       // this lane's keys: key_base .. key_base + 7
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            f32x4 st0 = f32x4{0.f, 0.f, 0.f, 0.f}, st1 = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) {
+                st0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(kf0[dc]), am_frag(qf[j][dc]), st0, 0, 0, 0);
+                st1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(kf1[dc]), am_frag(qf[j][dc]), st1, 0, 0, 0);
+            }
+            float sv[8];
+            float bmax = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int key = key_base + i;
+                const float raw = (i < 4) ? st0[i] : st1[i - 4];
+                sv[i] = (key <= p_col[j] && key >= lo_col[j]) ? raw * scale : -INFINITY;
+                bmax = fmaxf(bmax, sv[i]);
+            }
+            bmax = fmaxf(bmax, __shfl_xor(bmax, 16, TL_WAVE));
+            bmax = fmaxf(bmax, __shfl_xor(bmax, 32, TL_WAVE));
+            const float m_new = fmaxf(m_run[j], bmax);
+            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = expf(m_run[j] - m_safe);
+            float pr[8], psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                pr[i] = expf(sv[i] - m_safe);
+                psum += pr[i];
+            }
+            l_run[j] = l_run[j] * alpha + psum;
+            m_run[j] = m_new;
+            uint4 pf;
+            pf.x = am_pack2(pr[0], pr[1]);
+            pf.y = am_pack2(pr[2], pr[3]);
+            pf.z = am_pack2(pr[4], pr[5]);
+            pf.w = am_pack2(pr[6], pr[7]);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                f32x4 a = acc[j][db];
+                a[0] *= alpha;
+                a[1] *= alpha;
+                a[2] *= alpha;
+                a[3] *= alpha;
+                acc[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(vf[db]), am_frag(pf), a, 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- write: accumulator register i of lane (c, g) is (dim db*16 + 4g + i, column c) ----
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        if (p_col[j] < 0) continue;
+        float l_tot = l_run[j];
+        l_tot += __shfl_xor(l_tot, 16, TL_WAVE);
+        l_tot += __shfl_xor(l_tot, 32, TL_WAVE);
+        if (nsplit == 1) {
+            const float inv = 1.0f / l_tot;
+            bf16_t* op = out + (size_t)row_col[j] * out_stride + (size_t)head_col[j] * D + 4 * g;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                uint2 w;
+                w.x = am_pack2(acc[j][db][0] * inv, acc[j][db][1] * inv);
+                w.y = am_pack2(acc[j][db][2] * inv, acc[j][db][3] * inv);
+                *reinterpret_cast<uint2*>(op + db * 16) = w;
+            }
+        } else {
+            const size_t part = ((size_t)row_col[j] * nq + head_col[j]) * nsplit + sp;
+            float* wp = ws_o + part * D + 4 * g;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                *reinterpret_cast<f32x4*>(wp + db * 16) = acc[j][db];
+            if (g == 0) {
+                ws_ml[part * 2] = m_run[j];
+                ws_ml[part * 2 + 1] = l_tot;
+            }
+        }
+    }
+}
+
+// Merge the splits of one (token, head): M = max m_s, out = sum acc_s e^(m_s - M) / sum l_s e^(m_s - M),
+// over the splits that hold keys of the token, in ascending order.
+__global__ void attn_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+                                  const int32_t* __restrict__ pos, bf16_t* __restrict__ out, int out_stride, int nq,
+                                  int D, int nsplit, int split_blocks, int window) {
+    const int t = blockIdx.x, h = blockIdx.y;
+    const int p = pos[t];
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int s_lo = (lo >> 5) / split_blocks, s_hi = (p >> 5) / split_blocks;
+    const size_t base = ((size_t)t * nq + h) * nsplit;
+    float M = -INFINITY;
+    for (int s = s_lo; s <= s_hi; ++s) M = fmaxf(M, ws_ml[(base + s) * 2]);
+    float L = 0.f;
+    for (int s = s_lo; s <= s_hi; ++s) {
+        const float ms = ws_ml[(base + s) * 2];
+        if (ms > -INFINITY) L += ws_ml[(base + s) * 2 + 1] * expf(ms - M);
+    }
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float o = 0.f;
+        for (int s = s_lo; s <= s_hi; ++s) {
+            const float ms = ws_ml[(base + s) * 2];
+            if (ms > -INFINITY) o += ws_o[(base + s) * D + d] * expf(ms - M);
+        }
+        out[(size_t)t * out_stride + (size_t)h * D + d] = tl_from_float<bf16_t>(o / L);
+    }
+}
+
+template <int DC>
+static void launch_attn(int NT, dim3 grid, hipStream_t stream, const bf16_t* q, int q_stride, const bf16_t* kc,
+                        const bf16_t* vc, const int32_t* tables, int NB, const int32_t* q_start,
+                        const int32_t* ctx_start, bf16_t* out, int out_stride, float* ws_o, float* ws_ml, int nq, int nkv,
+                        int bs, int window, float scale, int nsplit, int split_blocks) {
+    if (NT == 1)
+        hipLaunchKernelGGL((attn_mfma_kernel<DC, 1>), grid, dim3(256), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
+                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+    else
+        hipLaunchKernelGGL((attn_mfma_kernel<DC, 2>), grid, dim3(256), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
+                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+}
+
+// q: bfloat16 [T, >= nq*d] (row stride q_stride); k_cache [pages, page, nkv, d]; v_cache
+// [pages, nkv, d, page]; tables int32 [S, NB]; q_start int32 [S+1]; ctx_start int32 [S]; out
+// bfloat16 [T, nq*d] (row stride out_stride).  NT (1 or 2) column tiles per wave; max_tile_groups =
+// the largest ceil(n_s * G / (16 NT)) over the sequences.  With nsplit > 1 a split is split_blocks
+// blocks of 32 keys, nsplit * split_blocks * 32 must cover the longest context, pos is int32 [T]
+// (the tokens' positions), ws_o holds T*nq*nsplit*d floats and ws_ml T*nq*nsplit*2.
+extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                 const int32_t* tables, int NB, const int32_t* q_start, const int32_t* ctx_start,
+                                 const int32_t* pos, void* out, int out_stride, float* ws_o, float* ws_ml, int T, int S,
+                                 int nq, int nkv, int d, int bs, int window, float scale, int NT, int max_tile_groups,
+                                 int nsplit, int split_blocks, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && NB > 0, "tl_attention_mfma: bad sizes T=%d S=%d nq=%d nkv=%d NB=%d", T, S, nq, nkv, NB);
+    TL_CHECK_ARG(nq % nkv == 0, "tl_attention_mfma: %d query heads are not a multiple of %d key/value heads", nq, nkv);
+    TL_CHECK_ARG(d == 32 || d == 64 || d == 128, "tl_attention_mfma: head size %d is not one of 32, 64, 128", d);
+    TL_CHECK_ARG(bs >= 8 && bs % 8 == 0, "tl_attention_mfma: page size %d must be a multiple of 8", bs);
+    TL_CHECK_ARG(NT == 1 || NT == 2, "tl_attention_mfma: NT=%d must be 1 or 2", NT);
+    TL_CHECK_ARG(nsplit >= 1 && max_tile_groups >= 1, "tl_attention_mfma: bad split or group count");
+    TL_CHECK_ARG(nsplit == 1 || (ws_o && ws_ml && pos && split_blocks >= 1),
+                 "tl_attention_mfma: split keys need a workspace, positions and a split length");
+    TL_CHECK_ARG(q_stride % 8 == 0 && out_stride % 4 == 0 && q_stride >= nq * d && out_stride >= nq * d,
+                 "tl_attention_mfma: bad row strides %d, %d", q_stride, out_stride);
+    TL_CHECK_ARG(((uintptr_t)q % 16) == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0 &&
+                     ((uintptr_t)out % 8) == 0, "tl_attention_mfma: operands must be 16-byte aligned");
+    TL_CHECK_ARG(nkv <= 65535, "tl_attention_mfma: too many key/value heads");
+    if (T == 0 || S == 0) return 0;
+    const long waves = (long)max_tile_groups * nsplit;
+    TL_CHECK_ARG((waves + 3) / 4 <= 65535, "tl_attention_mfma: too many tile groups x splits (%ld)", waves);
+    dim3 grid(S, nkv, (unsigned)((waves + 3) / 4));
+    const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
+    if (d == 32)
+        launch_attn<1>(NT, grid, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+    else if (d == 64)
+        launch_attn<2>(NT, grid, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+    else
+        launch_attn<4>(NT, grid, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+    TL_CHECK_LAUNCH("tl_attention_mfma");
+    if (nsplit > 1) {
+        hipLaunchKernelGGL(attn_merge_kernel, dim3(T, nq), dim3(d < 64 ? 64 : d), 0, stream, ws_o, ws_ml, pos,
+                           (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window);
+        TL_CHECK_LAUNCH("tl_attention_mfma merge");
+    }
+    return 0;
+}

@@ -125,15 +125,17 @@ extern "C" int tl_add_rmsnorm(float* x, const void* residual, int res_dtype, con
 // ---- rotary position encoding + cache write ------------------------------------------------
 // qkv: [T, (nq + 2 nkv) * d] as the fused projection leaves it.  Query heads are rotated in place;
 // key heads are rotated and written to k_cache at the token's slot; value heads are copied to
-// v_cache.  Rotate-half layout over the first `rot` dims of a head (reference: fused.py:34-51):
+// v_cache, which is transposed within a page so that the keys of one page are contiguous for each
+// head dim (what the matrix cores want for the P*V product).  Rotate-half layout over the first `rot` dims of a head (reference: fused.py:34-51):
 //   out[i]         = a*cos(theta_i) - b*sin(theta_i)       a = x[i], b = x[i + rot/2]
 //   out[i + rot/2] = b*cos(theta_i) + a*sin(theta_i)       theta_i = pos * inv_freq[i]
 // The angle, sine and cosine are float.  A negative slot skips the cache write of that token.
-// Caches are [pages, page, nkv, d], addressed here as [slot, nkv, d].
+// k_cache is [pages, page, nkv, d] (addressed as [slot, nkv, d]); v_cache is [pages, nkv, d, page].
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict__ pos,
                                   const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                  const int32_t* __restrict__ slots, int nq, int nkv, int d, int rot, int write_kv) {
+                                  const int32_t* __restrict__ slots, int nq, int nkv, int d, int rot, int write_kv,
+                                  int bs) {
     const int t = blockIdx.x;
     const int half = rot / 2;
     const float p = (float)pos[t];
@@ -167,24 +169,25 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
     }
     // values
     const T* vrow = row + (size_t)(nq + nkv) * d;
-    T* vdst = v_cache + (size_t)slot * nkv * d;
-    for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x) vdst[idx] = vrow[idx];
+    const int page = slot / bs, off = slot - page * bs;
+    T* vdst = v_cache + (size_t)page * nkv * d * bs + off;
+    for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x) vdst[(size_t)idx * bs] = vrow[idx];
 }
 
 extern "C" int tl_rope_store(void* qkv, int dtype, const int32_t* pos, const float* inv_freq, void* k_cache,
                              void* v_cache, const int32_t* slots, int T, int nq, int nkv, int d, int rot,
-                             int write_kv, hipStream_t stream) {
+                             int write_kv, int bs, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && nq > 0 && nkv >= 0 && d > 0, "tl_rope_store: bad sizes T=%d nq=%d nkv=%d d=%d", T, nq, nkv, d);
     TL_CHECK_ARG(rot >= 0 && rot <= d && rot % 2 == 0, "tl_rope_store: rotary width %d must be even and <= head size %d", rot, d);
-    TL_CHECK_ARG(!write_kv || (k_cache && v_cache && slots), "tl_rope_store: cache write asked for without a cache");
+    TL_CHECK_ARG(!write_kv || (k_cache && v_cache && slots && bs > 0), "tl_rope_store: cache write asked for without a cache");
     if (T == 0) return 0;
     dim3 grid(T), block(256);
     if (dtype == TL_F32)
         hipLaunchKernelGGL(rope_store_kernel<float>, grid, block, 0, stream, (float*)qkv, pos, inv_freq,
-                           (float*)k_cache, (float*)v_cache, slots, nq, nkv, d, rot, write_kv);
+                           (float*)k_cache, (float*)v_cache, slots, nq, nkv, d, rot, write_kv, bs);
     else if (dtype == TL_BF16)
         hipLaunchKernelGGL(rope_store_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, pos, inv_freq,
-                           (bf16_t*)k_cache, (bf16_t*)v_cache, slots, nq, nkv, d, rot, write_kv);
+                           (bf16_t*)k_cache, (bf16_t*)v_cache, slots, nq, nkv, d, rot, write_kv, bs);
     else
         return tl_fail("tl_rope_store: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("tl_rope_store");

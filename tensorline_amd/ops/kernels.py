@@ -224,6 +224,17 @@ def swiglu_gate_up(h: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tenso
     return silu_mul(linear(h, gate_up_weight))
 
 
+def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, who: str) -> None:
+    """Keys are paged as [pages, page, nkv, d]; values as [pages, nkv, d, page] (transposed in the page)."""
+    _check(k_cache.dtype == dtype and k_cache.is_contiguous() and k_cache.dim() == 4
+           and k_cache.shape[2] == num_kv_heads and k_cache.shape[3] == head_dim,
+           f"{who}: key cache must be contiguous [pages, page, nkv, d] of the activation dtype")
+    pages, page = k_cache.shape[0], k_cache.shape[1]
+    _check(v_cache.dtype == dtype and v_cache.is_contiguous()
+           and tuple(v_cache.shape) == (pages, num_kv_heads, head_dim, page),
+           f"{who}: value cache must be contiguous [pages, nkv, d, page] matching the key cache")
+
+
 def rope_store(qkv: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor | None, num_heads: int,
                num_kv_heads: int, head_dim: int, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None,
                slots: torch.Tensor | None) -> None:
@@ -243,30 +254,33 @@ def rope_store(qkv: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor | No
     write = k_cache is not None
     if write:
         _check(v_cache is not None and slots is not None, "rope_store: cache write needs k_cache, v_cache and slots")
-        for c in (k_cache, v_cache):
-            _check(c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
-                   and c.shape[2] == num_kv_heads and c.shape[3] == head_dim,
-                   "rope_store: cache must be contiguous [pages, page, nkv, d] of the activation dtype")
+        _check_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim, "rope_store")
         _i32(slots, "slots", T)
     _call("tl_rope_store", _ptr(qkv), _code(qkv, "rope_store"), _ptr(pos), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache),
-          _ptr(slots), T, num_heads, num_kv_heads, head_dim, rot, 1 if write else 0, _stream())
+          _ptr(slots), T, num_heads, num_kv_heads, head_dim, rot, 1 if write else 0,
+          k_cache.shape[1] if write else 0, _stream())
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, tables: torch.Tensor,
                     seq_of_token: torch.Tensor, pos: torch.Tensor, num_heads: int, num_kv_heads: int,
                     head_dim: int, scale: float, window: int = 0, out: torch.Tensor | None = None,
-                    plan=None) -> torch.Tensor:
+                    q_start: torch.Tensor | None = None, ctx_start: torch.Tensor | None = None, plan=None,
+                    path: str | None = None, split_keys: int | None = None) -> torch.Tensor:
     """Causal attention of each token over the cached keys of its sequence.
 
     ``q``: [T, >= nq*d] with the query heads in the first nq*d columns (row stride free);
     ``tables``: int32 [S, NB] page ids; ``seq_of_token``, ``pos``: int32 [T].  ``window`` > 0
-    limits a token at position p to keys [p - window + 1, p].  Returns [T, nq*d]."""
-    _on_gpu(q, k_cache, v_cache, tables, seq_of_token, pos, out)
+    limits a token at position p to keys [p - window + 1, p].  Returns [T, nq*d].
+
+    bfloat16 with a head size of 32, 64 or 128 and pages of a multiple of 8 tokens runs on the
+    matrix cores; that kernel works per sequence and needs ``q_start`` [S+1], ``ctx_start`` [S]
+    and the host-side ``plan`` (lengths of the step's sequences).  Everything else runs the
+    any-shape kernel.  ``path`` ("mfma" or "generic") forces one of them; ``split_keys`` forces the
+    number of keys per split (0: no split)."""
+    _on_gpu(q, k_cache, v_cache, tables, seq_of_token, pos, out, q_start, ctx_start)
     T = q.shape[0]
     _check(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= num_heads * head_dim, "paged_attention: bad query layout")
-    for c in (k_cache, v_cache):
-        _check(c.dtype == q.dtype and c.is_contiguous() and c.dim() == 4 and c.shape[2] == num_kv_heads
-               and c.shape[3] == head_dim, "paged_attention: cache must be contiguous [pages, page, nkv, d]")
+    _check_caches(k_cache, v_cache, q.dtype, num_kv_heads, head_dim, "paged_attention")
     _check(tables.dim() == 2 and tables.dtype == torch.int32 and tables.is_contiguous(), "paged_attention: bad page table")
     _i32(seq_of_token, "seq_of_token", T)
     _i32(pos, "pos", T)
@@ -275,9 +289,48 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _check(out.dtype == q.dtype and out.dim() == 2 and out.shape[0] == T and out.stride(1) == 1, "paged_attention: bad output")
     q_stride = q.stride(0) if T > 1 else q.shape[1]
     o_stride = out.stride(0) if T > 1 else out.shape[1]
+    page = k_cache.shape[1]
+    mfma_ok = (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and page % 8 == 0 and q_start is not None
+               and ctx_start is not None and plan is not None and q_stride % 8 == 0 and o_stride % 4 == 0
+               and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0)
+    if path == "mfma":
+        _check(mfma_ok, "paged_attention: the matrix-core kernel does not take these arguments")
+    if mfma_ok and path != "generic":
+        S = tables.shape[0]
+        _i32(q_start, "q_start", S + 1)
+        _i32(ctx_start, "ctx_start", S)
+        G = num_heads // num_kv_heads
+        nt = 1 if plan.max_query_len * G <= 16 else 2
+        groups = [-(-n * G // (16 * nt)) for n in plan.q_lens]
+        pads = max(0, S - len(groups))                     # padding sequences bring one token each
+        max_groups = max(groups + [1])
+        # Splits are fixed runs of keys aligned to absolute positions, so the same keys are summed
+        # together whatever the context length or the launch shape.  Pure decode steps split by the
+        # batch size rounded up to a power of two (what a graph bucket pads to); steps with prompt
+        # portions have enough columns and do not split.
+        split_len = 0
+        if split_keys is not None:
+            split_len = int(split_keys)
+        elif plan.decode_only:
+            base = (1 << max(S - 1, 0).bit_length()) * num_kv_heads
+            split_len = 64 if base <= 8 else 128 if base <= 32 else 256 if base <= 128 else 512 if base <= 512 else 0
+        nsplit, split_blocks = 1, 1
+        if split_len:
+            _check(split_len % 32 == 0, "paged_attention: a split is a multiple of 32 keys")
+            split_blocks = split_len // 32
+            nsplit = max(1, -(-plan.max_context // split_len))
+        ws_o = ws_ml = None
+        if nsplit > 1:
+            ws = torch.empty(T * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
+            ws_o, ws_ml = ws[:T * num_heads * nsplit * head_dim], ws[T * num_heads * nsplit * head_dim:]
+        _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
+              _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,
+              num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,
+              _stream())
+        return out
     _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
           _ptr(seq_of_token), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, num_heads,
-          num_kv_heads, head_dim, k_cache.shape[1], int(window), ctypes.c_float(scale), _stream())
+          num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), _stream())
     return out
 
 

@@ -77,5 +77,6 @@ class PagedAttention(Part):
                                       cache.slots if write else None)
         o = kernels.paged_attention(qkv, cache.k, cache.v, cache.tables, ctx.seq_of_token, ctx.pos,
                                     self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
-                                    window=self.window, plan=ctx.attention_plan)
+                                    window=self.window, q_start=ctx.q_start, ctx_start=ctx.ctx_start,
+                                    plan=ctx.attention_plan)
         return self.o_proj(o, out_dtype=torch.float32)

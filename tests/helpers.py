@@ -20,8 +20,12 @@ TINY_B = dict(architectures=["Qwen2ForCausalLM"], vocab_size=1000, hidden_size=1
 TINY_C = dict(architectures=["Qwen2ForCausalLM"], vocab_size=777, hidden_size=120, intermediate_size=200,
               num_hidden_layers=2, num_attention_heads=5, num_key_value_heads=1, head_dim=48,
               rope_theta=50000.0, rms_norm_eps=3e-6, tie_word_embeddings=False, max_position_embeddings=1024)
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-PAGE = {"A": 16, "B": 8, "C": 16}
+# One with the head size of the large models (128), heads wider than the hidden size, group 3.
+TINY_D = dict(architectures=["Qwen2ForCausalLM"], vocab_size=2000, hidden_size=256, intermediate_size=368,
+              num_hidden_layers=2, num_attention_heads=6, num_key_value_heads=2, head_dim=128,
+              rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=2048)
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+PAGE = {"A": 16, "B": 8, "C": 16, "D": 16}
 
 
 def make_model_dir(tmp_path_factory_or_dir, name: str, seed: int = 0) -> str:

@@ -56,17 +56,20 @@ def rope_store(qkv, pos, inv_freq, num_heads, num_kv_heads, head_dim, k_cache, v
     heads[:, :num_heads] = rot_heads[:, :num_heads]
     if k_cache is not None:
         ok = slots >= 0
-        kc, vc = k_cache.view(-1, num_kv_heads, d), v_cache.view(-1, num_kv_heads, d)
+        bs = k_cache.shape[1]
+        kc = k_cache.view(-1, num_kv_heads, d)
         kc[slots[ok].long()] = rot_heads[ok][:, num_heads:]
-        vc[slots[ok].long()] = heads[ok][:, num_heads + num_kv_heads:]
+        sl = slots[ok].long()
+        v_cache[sl // bs, :, :, sl % bs] = heads[ok][:, num_heads + num_kv_heads:]      # [pages, nkv, d, page]
 
 
 def paged_attention(q, k_cache, v_cache, tables, seq_of_token, pos, num_heads, num_kv_heads, head_dim, scale,
-                    window=0, out=None, plan=None):
+                    window=0, out=None, q_start=None, ctx_start=None, plan=None, path=None, split_keys=None):
     T, d, bs = q.shape[0], head_dim, k_cache.shape[1]
     g = num_heads // num_kv_heads
     o = torch.empty(T, num_heads * d, dtype=q.dtype)
-    kc, vc = k_cache.view(-1, num_kv_heads, d), v_cache.view(-1, num_kv_heads, d)
+    kc = k_cache.view(-1, num_kv_heads, d)
+    vc = v_cache.permute(0, 3, 1, 2).reshape(-1, num_kv_heads, d)                      # back to [slot, nkv, d]
     for t in range(T):
         s, p = int(seq_of_token[t]), int(pos[t])
         lo = max(0, p - window + 1) if window > 0 else 0

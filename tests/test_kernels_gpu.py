@@ -130,7 +130,7 @@ def test_rope_store(dtype, nq, nkv, d, rot):
     slots = torch.randperm(pages * bs, device=DEV)[:T].to(torch.int32)
     slots[5] = -1
     kc = torch.full((pages, bs, nkv, d), 7.0, device=DEV).to(dtype)
-    vc = torch.full((pages, bs, nkv, d), 7.0, device=DEV).to(dtype)
+    vc = torch.full((pages, nkv, d, bs), 7.0, device=DEV).to(dtype)       # values: transposed within the page
     i = torch.arange(0, rot, 2, dtype=torch.float64)
     inv_freq = (theta ** (-i / rot)).float().to(DEV)
     heads = qkv.float().cpu().view(T, nq + 2 * nkv, d)
@@ -141,7 +141,7 @@ def test_rope_store(dtype, nq, nkv, d, rot):
     got = qkv.float().cpu().view(T, nq + 2 * nkv, d)
     t = tol(dtype, 2e-5, 2e-2)
     torch.testing.assert_close(got[:, :nq], want_q, **t)
-    kf, vf = kc.float().cpu().view(-1, nkv, d), vc.float().cpu().view(-1, nkv, d)
+    kf, vf = kc.float().cpu().view(-1, nkv, d), vc.float().cpu().permute(0, 3, 1, 2).reshape(-1, nkv, d)
     ok = slots.cpu() >= 0
     torch.testing.assert_close(kf[slots.cpu()[ok].long()], want_k[ok], **t)
     torch.testing.assert_close(vf[slots.cpu()[ok].long()], want_v[ok], atol=0, rtol=0)
@@ -155,7 +155,7 @@ def test_rope_store(dtype, nq, nkv, d, rot):
     torch.testing.assert_close(qkv0, keep, atol=0, rtol=0)
 
 
-def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False):
+def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False, path=None, split_keys=None):
     """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries."""
     torch.manual_seed(seed)
     S = len(lens)
@@ -163,7 +163,7 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
     nb = max(-(-n // bs) for n in lens)
     num_blocks = S * nb + 8
     kc = torch.randn(num_blocks, bs, nkv, d, device=DEV).to(dtype)
-    vc = torch.randn(num_blocks, bs, nkv, d, device=DEV).to(dtype)
+    vc = torch.randn(num_blocks, nkv, d, bs, device=DEV).to(dtype)
     tables = torch.randperm(num_blocks, device=DEV)[:S * nb].view(S, nb).to(torch.int32)   # scattered pages
     seq_of, pos = [], []
     for s, (n, ql) in enumerate(zip(lens, q_lens)):
@@ -180,9 +180,18 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
             far = 1 if lens[s] > 2 else 0
             row = int(tables[s, far // bs]) * bs + far % bs
             kflat[row] = (q[t].view(nq, d)[:nkv].float() * 4).to(dtype)
+    from tensorline_amd.engine.batch import AttentionPlan
+    qs = [0]
+    for ql in q_lens:
+        qs.append(qs[-1] + ql)
+    plan = AttentionPlan(max_context=max(lens), max_query_len=max(q_lens), decode_only=max(q_lens) == 1,
+                         num_seqs=S, q_lens=list(q_lens), starts=[n - ql for n, ql in zip(lens, q_lens)])
     out = K().paged_attention(q, kc, vc, tables, torch.tensor(seq_of, dtype=torch.int32, device=DEV),
-                              torch.tensor(pos, dtype=torch.int32, device=DEV), nq, nkv, d, d ** -0.5, window=window)
-    kf, vf = kc.double().cpu().view(-1, nkv, d), vc.double().cpu().view(-1, nkv, d)
+                              torch.tensor(pos, dtype=torch.int32, device=DEV), nq, nkv, d, d ** -0.5, window=window,
+                              q_start=torch.tensor(qs, dtype=torch.int32, device=DEV),
+                              ctx_start=torch.tensor(plan.starts, dtype=torch.int32, device=DEV), plan=plan,
+                              path=path, split_keys=split_keys)
+    kf, vf = kc.double().cpu().view(-1, nkv, d), vc.double().cpu().permute(0, 3, 1, 2).reshape(-1, nkv, d)
     want = torch.empty(T, nq, d, dtype=torch.float64)
     tcpu = tables.cpu().long()
     t0 = 0
@@ -212,6 +221,31 @@ def test_attention_portions_and_spike(dtype, nq, nkv, d, bs):
     torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
 
 
+@pytest.mark.parametrize("path", ["generic", "mfma"])
+@pytest.mark.parametrize("heads", [(14, 2), (12, 2), (16, 2), (4, 4), (28, 4)])
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_attention_matrix_core_kernel(path, heads, d):
+    """The matrix-core kernel against the plain attention: decode rows and prompt portions in one
+    batch, scattered pages, a key that dominates, contexts around block and page edges, and the
+    key range split 1, 3 and many ways."""
+    dtype = torch.bfloat16
+    lens = [1, 31, 32, 33, 65, 300, 1400, 2, 129]
+    q_lens = [1, 1, 32, 5, 64, 1, 9, 2, 100]
+    for split_keys in (0, 32, 96, None):
+        got, want = _attention_case(dtype, heads[0], heads[1], d, 16, lens, q_lens, seed=7, spike=True, path=path,
+                                    split_keys=split_keys)
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+    lens = [63, 64, 65, 300, 1400, 1400, 17]                  # decode only, page of 8
+    for split_keys in (0, 64, 256, None):
+        got, want = _attention_case(dtype, heads[0], heads[1], d, 8, lens, seed=8, path=path, split_keys=split_keys)
+        torch.testing.assert_close(got, want, atol=1e-2, rtol=1e-2)
+    for window in (1, 7, 32, 100):
+        for split_keys in (0, 64):
+            got, want = _attention_case(dtype, heads[0], heads[1], d, 16, [50, 7, 130, 700], [20, 7, 1, 33],
+                                        window=window, seed=9, path=path, split_keys=split_keys)
+            torch.testing.assert_close(got, want, atol=1e-2, rtol=1e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("window", [1, 7, 16, 100])
 def test_attention_window(dtype, window):
@@ -223,15 +257,15 @@ def test_attention_special_cases():
     # one key: o = v;  q = 0: o = mean of the visible values
     dtype, nq, nkv, d, bs = torch.float32, 4, 2, 16, 8
     kc = torch.randn(4, bs, nkv, d, device=DEV)
-    vc = torch.randn(4, bs, nkv, d, device=DEV)
+    vc = torch.randn(4, nkv, d, bs, device=DEV)
     tables = torch.tensor([[2, 0]], dtype=torch.int32, device=DEV)
     z = torch.zeros(1, dtype=torch.int32, device=DEV)
     q = torch.randn(1, nq * d, device=DEV)
     o = K().paged_attention(q, kc, vc, tables, z, z, nq, nkv, d, 0.25).view(nq, d)
-    torch.testing.assert_close(o, vc[2, 0].repeat_interleave(2, 0), atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(o, vc[2, :, :, 0].repeat_interleave(2, 0), atol=1e-6, rtol=1e-6)
     p = torch.tensor([10], dtype=torch.int32, device=DEV)
     o = K().paged_attention(torch.zeros_like(q), kc, vc, tables, z, p, nq, nkv, d, 0.25).view(nq, d)
-    vis = torch.cat([vc[2], vc[0, :3]]).mean(0)
+    vis = torch.cat([vc[2].permute(2, 0, 1), vc[0].permute(2, 0, 1)[:3]]).mean(0)
     torch.testing.assert_close(o, vis.repeat_interleave(2, 0), atol=1e-6, rtol=1e-6)
 
 
@@ -316,6 +350,6 @@ def test_bad_arguments_are_refused():
         K().add_rmsnorm(torch.randn(2, 8), None, torch.ones(8), 1e-6, torch.float32)
     with pytest.raises(KernelError):
         kc = torch.randn(2, 4, 1, 512, device=DEV)
-        K().paged_attention(torch.randn(1, 512, device=DEV), kc, kc, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+        K().paged_attention(torch.randn(1, 512, device=DEV), kc, kc.permute(0, 2, 3, 1).contiguous(), torch.zeros(1, 1, dtype=torch.int32, device=DEV),
                             torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
                             1, 1, 512, 1.0)

@@ -14,12 +14,12 @@ from tests import helpers, plain
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LENGTHS = {"A": [5, 17, 33, 70, 130], "B": [1, 8, 31, 64, 100, 300], "C": [2, 40, 65, 257]}
+LENGTHS = {"A": [5, 17, 33, 70, 130], "B": [1, 8, 31, 64, 100, 300], "C": [2, 40, 65, 257], "D": [3, 64, 97, 600]}
 # error of the logits relative to the largest logit of the request
-LIMIT = {"float32": 5e-5, "bfloat16": 3e-2}
+LIMIT = {"float32": 1e-5, "bfloat16": 2e-2}
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D"])
 def setup(request, tmp_path_factory):
     name = request.param
     d = helpers.make_model_dir(tmp_path_factory, name, seed=5)
