@@ -12,6 +12,7 @@ from typing import Callable
 import torch
 
 from tensorline_amd.ops import kernels
+from tensorline_amd.parts.base import Linear
 from tensorline_amd.parts.registry import BLOCKS, build_part, _ensure_builtin
 from tensorline_amd.parts.spec import CacheNeed, ModelSpec, StateNeed, TensorDecl
 
@@ -38,7 +39,7 @@ class DecoderModel:
         self.head_name = spec.head.params["name"]
         self.tied = bool(spec.head.params.get("tied", False))
         self.embed_table: torch.Tensor | None = None
-        self.head_weight: torch.Tensor | None = None
+        self.head = Linear(self.head_name.removesuffix(".weight"), spec.hidden_size, spec.vocab_size, False)
 
     # ---- weights -----------------------------------------------------------------------
     def tensor_decls(self) -> dict[str, TensorDecl]:
@@ -62,12 +63,13 @@ class DecoderModel:
             for p in b.parts():
                 p.load(get)
         self.final_norm.load(get)
-        self.head_weight = self.embed_table if self.tied else get(self.head_name)
+        self.head.weight = self.embed_table if self.tied else get(self.head_name)
+        self.head.prepare()
 
     def weight_bytes(self) -> int:
         """Bytes of weights on the device, a shared tensor counted once (reference: quant.py:107-113)."""
         seen, total = set(), 0
-        tensors = [self.embed_table, self.head_weight] + self.final_norm.weight_tensors()
+        tensors = [self.embed_table] + self.head.tensors_kept() + self.final_norm.weight_tensors()
         for b in self.blocks:
             for p in b.parts():
                 tensors += p.weight_tensors()
@@ -107,4 +109,4 @@ class DecoderModel:
             # the residual stream is complete only after the last add; nothing reads it here
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=x.device)
         h = self.final_norm.forward(x, pending, rows=ctx.logit_rows)
-        return kernels.linear(h, self.head_weight, None, out_dtype=torch.float32)
+        return self.head(h, out_dtype=torch.float32)

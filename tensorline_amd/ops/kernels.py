@@ -139,10 +139,35 @@ def add_rmsnorm(x: torch.Tensor, residual: torch.Tensor | None, weight: torch.Te
     return out
 
 
+def shuffle_weight(weight: torch.Tensor) -> torch.Tensor | None:
+    """The copy of a bfloat16 [N, K] matrix that the few-row kernel streams: [ceil(N/16) tiles,
+    ceil(K/32) chunks, 64 lanes, 8 values], lane 16*g + r holding row r of the tile at k = 32*chunk +
+    8*g .. +8, zero where it pads.  None for matrices that kernel does not take."""
+    if weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.shape[1] % 8:
+        return None
+    N, K = weight.shape
+    Np, Kp = -(-N // 16) * 16, -(-K // 32) * 32
+    if (Np, Kp) != (N, K):
+        padded = torch.zeros(Np, Kp, dtype=weight.dtype, device=weight.device)
+        padded[:N, :K] = weight
+    else:
+        padded = weight
+    return padded.view(Np // 16, 16, Kp // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+
+
+def _check_shuffled(shuffled: torch.Tensor, N: int, K: int) -> None:
+    _check(shuffled.dtype == torch.bfloat16 and shuffled.is_contiguous()
+           and tuple(shuffled.shape) == (-(-N // 16), -(-K // 32), 4, 16, 8),
+           f"linear: the shuffled weight copy does not belong to a [{N}, {K}] matrix")
+
+
 def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
-           out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
-    """``a @ weight.T + bias``: a [M, K] (rows may be strided), weight [N, K], bias float32 [N]."""
-    _on_gpu(a, weight, bias, out)
+           out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
+           shuffled: torch.Tensor | None = None) -> torch.Tensor:
+    """``a @ weight.T + bias``: a [M, K] (rows may be strided), weight [N, K], bias float32 [N].
+    ``shuffled``: the copy of ``weight`` made by :func:`shuffle_weight`, which few-row bfloat16
+    products stream instead of ``weight``."""
+    _on_gpu(a, weight, bias, out, shuffled)
     _check(a.dim() == 2 and a.stride(1) == 1, "linear: input must be [M, K] with unit column stride")
     _check(weight.dim() == 2 and weight.is_contiguous(), "linear: weight must be a contiguous [N, K] matrix")
     M, K = a.shape
@@ -160,23 +185,25 @@ def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
            "linear: bad output")
     lda = a.stride(0) if M > 1 else K
     ldc = out.stride(0) if M > 1 else N
-    return _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc)
+    if shuffled is not None:
+        _check_shuffled(shuffled, N, K)
+    return _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled)
 
 
 SKINNY_MAX_ROWS = 64
 
 
-def _skinny_ok(a: torch.Tensor, weight: torch.Tensor, M: int, K: int, lda: int) -> bool:
-    return (a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS
-            and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+def _skinny_ok(a: torch.Tensor, shuffled: torch.Tensor | None, M: int, K: int, lda: int) -> bool:
+    return (shuffled is not None and a.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS
+            and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0)
 
 
-def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc) -> torch.Tensor:
+def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled=None) -> torch.Tensor:
     """bfloat16 with few rows: the streaming MFMA kernel.  float32, and shapes that kernel does not
     take: the plain tiled kernel.  (bfloat16 with many rows went to the library before this, where
     the reference uses one too: tensorline/paged.py:179-188.)"""
-    if _skinny_ok(a, weight, M, K, lda):
-        _call("tl_gemm_skinny", _ptr(a), _ptr(weight), _ptr(bias), _ptr(out), _code(out, "linear output"),
+    if _skinny_ok(a, shuffled, M, K, lda):
+        _call("tl_gemm_skinny", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), _code(out, "linear output"),
               M, N, K, lda, ldc, _stream())
         return out
     _call("tl_gemm_generic", _ptr(a), _code(a, "linear input"), _ptr(weight), _code(weight, "linear weight"),
@@ -208,20 +235,22 @@ def _library_linear(a, weight, bias, out_dtype) -> torch.Tensor:
     return y
 
 
-def swiglu_gate_up(h: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+def swiglu_gate_up(h: torch.Tensor, gate_up_weight: torch.Tensor, shuffled: torch.Tensor | None = None) -> torch.Tensor:
     """``silu(h Wg^T) * (h Wu^T)`` for a fused [2I, K] weight (gate rows first): one kernel for
-    few-row bfloat16 batches, product then SiLU-multiply otherwise."""
-    _on_gpu(h, gate_up_weight)
+    few-row bfloat16 batches (it streams the ``shuffled`` copy), product then SiLU-multiply otherwise."""
+    _on_gpu(h, gate_up_weight, shuffled)
     _check(h.dim() == 2 and h.stride(1) == 1 and gate_up_weight.dim() == 2 and gate_up_weight.is_contiguous()
            and gate_up_weight.shape[0] % 2 == 0 and gate_up_weight.shape[1] == h.shape[1], "swiglu_gate_up: bad shapes")
     M, K = h.shape
     I = gate_up_weight.shape[0] // 2
     lda = h.stride(0) if M > 1 else K
-    if _skinny_ok(h, gate_up_weight, M, K, lda):
+    if shuffled is not None:
+        _check_shuffled(shuffled, 2 * I, K)
+    if _skinny_ok(h, shuffled, M, K, lda) and I % 16 == 0:
         out = torch.empty(M, I, dtype=h.dtype, device=h.device)
-        _call("tl_gemm_skinny_swiglu", _ptr(h), _ptr(gate_up_weight), _ptr(out), M, I, K, lda, I, _stream())
+        _call("tl_gemm_skinny_swiglu", _ptr(h), _ptr(shuffled), _ptr(out), M, I, K, lda, I, _stream())
         return out
-    return silu_mul(linear(h, gate_up_weight))
+    return silu_mul(linear(h, gate_up_weight, shuffled=shuffled))
 
 
 def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, who: str) -> None:

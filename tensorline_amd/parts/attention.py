@@ -56,9 +56,10 @@ class PagedAttention(Part):
         for p in self._projs:          # the fused copy is the one that is kept
             p.weight = p.bias = None
         self.o_proj.load(get)
+        self.o_proj.prepare()
 
     def weight_tensors(self):
-        return [t for t in (self.qkv.weight, self.qkv.bias, self.o_proj.weight, self.o_proj.bias) if t is not None]
+        return self.qkv.tensors_kept() + self.o_proj.tensors_kept()
 
     # ---- what it keeps -------------------------------------------------------------------
     def cache_need(self) -> CacheNeed | None:

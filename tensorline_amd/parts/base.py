@@ -43,6 +43,7 @@ class Linear:
         self.in_features, self.out_features, self.has_bias, self.std = in_features, out_features, bias, std
         self.weight: torch.Tensor | None = None
         self.bias: torch.Tensor | None = None
+        self.shuffled: torch.Tensor | None = None     # the copy few-row bfloat16 products stream
 
     def tensors(self) -> dict[str, TensorDecl]:
         out = {self.name + ".weight": TensorDecl((self.out_features, self.in_features), "normal", self.std, "compute")}
@@ -54,8 +55,18 @@ class Linear:
         self.weight = get(self.name + ".weight")
         self.bias = get(self.name + ".bias") if self.has_bias else None
 
+    def prepare(self) -> "Linear":
+        """Make the second, matrix-core ordered copy of a bfloat16 weight.  Decode steps stream
+        that copy, many-row steps hand the row-major one to the library: twice the bytes, for
+        which 288 GB of HBM has room."""
+        self.shuffled = kernels.shuffle_weight(self.weight)
+        return self
+
+    def tensors_kept(self) -> list[torch.Tensor]:
+        return [t for t in (self.weight, self.bias, self.shuffled) if t is not None]
+
     def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        return kernels.linear(x, self.weight, self.bias, out_dtype=out_dtype)
+        return kernels.linear(x, self.weight, self.bias, out_dtype=out_dtype, shuffled=self.shuffled)
 
 
 def fuse_linears(name: str, parts: list[Linear]) -> Linear:
@@ -67,4 +78,4 @@ def fuse_linears(name: str, parts: list[Linear]) -> Linear:
         fused.bias = torch.cat([
             p.bias if p.bias is not None else torch.zeros(p.out_features, dtype=torch.float32, device=p.weight.device)
             for p in parts]).contiguous()
-    return fused
+    return fused.prepare()

@@ -32,10 +32,11 @@ class SwiGLU(Part):
         self.gate_up = fuse_linears(self.prefix + "gate_up_proj", [self._gate, self._up])
         self._gate.weight = self._up.weight = None
         self.down.load(get)
+        self.down.prepare()
 
     def weight_tensors(self):
-        return [self.gate_up.weight, self.down.weight]
+        return self.gate_up.tensors_kept() + self.down.tensors_kept()
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
-        act = kernels.swiglu_gate_up(h, self.gate_up.weight)
+        act = kernels.swiglu_gate_up(h, self.gate_up.weight, self.gate_up.shuffled)
         return self.down(act, out_dtype=torch.float32)

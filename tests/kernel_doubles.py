@@ -33,7 +33,11 @@ def add_rmsnorm(x, residual, weight, eps, out_dtype, rows=None, out=None):
     return r.to(out_dtype)
 
 
-def linear(a, weight, bias=None, out_dtype=None, out=None):
+def shuffle_weight(weight):
+    return None
+
+
+def linear(a, weight, bias=None, out_dtype=None, out=None, shuffled=None):
     y = a.to(torch.float32) @ weight.to(torch.float32).T
     if bias is not None:
         y = y + bias
@@ -89,7 +93,7 @@ def silu_mul(gate_up, out=None):
     return (g * torch.sigmoid(g) * u).to(gate_up.dtype)
 
 
-def swiglu_gate_up(h, gate_up_weight):
+def swiglu_gate_up(h, gate_up_weight, shuffled=None):
     return silu_mul(linear(h, gate_up_weight))
 
 
@@ -117,7 +121,7 @@ def sample(logits, temperature, top_p, uniform, out=None):
     return res
 
 
-ALL = ["require_gpu", "embed", "add_rmsnorm", "linear", "rope_store", "paged_attention", "silu_mul", "swiglu_gate_up", "argmax",
+ALL = ["require_gpu", "embed", "add_rmsnorm", "linear", "rope_store", "paged_attention", "silu_mul", "swiglu_gate_up", "shuffle_weight", "argmax",
        "sample"]
 
 
