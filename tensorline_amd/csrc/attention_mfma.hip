@@ -106,27 +106,34 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     }
 
     const int krow_in_block0 = 8 * (c >> 2) + (c & 3);         // key of row c in tile 0; tile 1: + 4
+    // One block ahead: while block b is multiplied, the fragments of block b + 1 are in flight
+    // (past the last block the same block is requested again and not used).
+    uint4 kf0[DC], kf1[DC], vf[DB], kn0[DC], kn1[DC], vn[DB];
+#define AM_LOAD_BLOCK(B, K0, K1, V)                                                                          \
+    {                                                                                                        \
+        const int kb_ = (B) << 5;                                                                            \
+        /* keys past khi are masked for every column; their addresses are clamped to stay on pages the */    \
+        /* sequence owns */                                                                                  \
+        int k0_ = kb_ + krow_in_block0, k1_ = k0_ + 4;                                                       \
+        if (k0_ > khi) k0_ = khi;                                                                            \
+        if (k1_ > khi) k1_ = khi;                                                                            \
+        const bf16_t* kp0_ = kc + ((size_t)(table[k0_ / bs] * bs + k0_ % bs) * nkv + kvh) * D + g * 8;       \
+        const bf16_t* kp1_ = kc + ((size_t)(table[k1_ / bs] * bs + k1_ % bs) * nkv + kvh) * D + g * 8;       \
+        _Pragma("unroll") for (int dc = 0; dc < DC; ++dc) {                                                  \
+            K0[dc] = *reinterpret_cast<const uint4*>(kp0_ + dc * 32);                                        \
+            K1[dc] = *reinterpret_cast<const uint4*>(kp1_ + dc * 32);                                        \
+        }                                                                                                    \
+        int vk_ = kb_ + 8 * g;                                                                               \
+        if (vk_ > khi) vk_ = khi & ~7;                                                                       \
+        const bf16_t* vp_ = vc + (((size_t)table[vk_ / bs] * nkv + kvh) * D + c) * bs + vk_ % bs;            \
+        _Pragma("unroll") for (int db = 0; db < DB; ++db)                                                    \
+            V[db] = *reinterpret_cast<const uint4*>(vp_ + (size_t)db * 16 * bs);                             \
+    }
+    AM_LOAD_BLOCK(bb, kf0, kf1, vf)
     for (int b = bb; b < be; ++b) {
         const int kb = b << 5;
-        // keys past khi are masked for every column; their addresses are clamped to stay on
-        // pages the sequence owns
-        int k0 = kb + krow_in_block0, k1 = k0 + 4;
-        if (k0 > khi) k0 = khi;
-        if (k1 > khi) k1 = khi;
-        const bf16_t* kp0 = kc + ((size_t)(table[k0 / bs] * bs + k0 % bs) * nkv + kvh) * D + g * 8;
-        const bf16_t* kp1 = kc + ((size_t)(table[k1 / bs] * bs + k1 % bs) * nkv + kvh) * D + g * 8;
-        uint4 kf0[DC], kf1[DC];
-#pragma unroll
-        for (int dc = 0; dc < DC; ++dc) {
-            kf0[dc] = *reinterpret_cast<const uint4*>(kp0 + dc * 32);
-            kf1[dc] = *reinterpret_cast<const uint4*>(kp1 + dc * 32);
-        }
-        int vk = kb + 8 * g;
-        if (vk > khi) vk = khi & ~7;
-        const bf16_t* vp = vc + (((size_t)table[vk / bs] * nkv + kvh) * D + c) * bs + vk % bs;
-        uint4 vf[DB];
-#pragma unroll
-        for (int db = 0; db < DB; ++db) vf[db] = *reinterpret_cast<const uint4*>(vp + (size_t)db * 16 * bs);
+        const int b_next = (b + 1 < be) ? b + 1 : b;
+        AM_LOAD_BLOCK(b_next, kn0, kn1, vn)
 
         const int key_base = kb + 8 * g;                       // this lane's keys: key_base .. key_base + 7
 #pragma unroll
@@ -174,8 +181,16 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
                 acc[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(vf[db]), am_frag(pf), a, 0, 0, 0);
             }
         }
+    #pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+            kf0[dc] = kn0[dc];
+            kf1[dc] = kn1[dc];
+        }
+#pragma unroll
+        for (int db = 0; db < DB; ++db) vf[db] = vn[db];
     }
 
+#undef AM_LOAD_BLOCK
     // ---- write: accumulator register i of lane (c, g) is (dim db*16 + 4g + i, column c) ----
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -209,28 +224,37 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
 
 // Merge the splits of one (token, head): M = max m_s, out = sum acc_s e^(m_s - M) / sum l_s e^(m_s - M),
 // over the splits that hold keys of the token, in ascending order.
+#define AM_MAX_SPLITS 256
 __global__ void attn_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                   const int32_t* __restrict__ pos, bf16_t* __restrict__ out, int out_stride, int nq,
                                   int D, int nsplit, int split_blocks, int window) {
+    __shared__ float wgt[AM_MAX_SPLITS];
+    __shared__ float inv_l;
     const int t = blockIdx.x, h = blockIdx.y;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int s_lo = (lo >> 5) / split_blocks, s_hi = (p >> 5) / split_blocks;
-    const size_t base = ((size_t)t * nq + h) * nsplit;
+    const int ns = s_hi - s_lo + 1;
+    const size_t base = ((size_t)t * nq + h) * nsplit + s_lo;
+    // every thread finds the maximum (a few cached loads), one thread per split its weight
     float M = -INFINITY;
-    for (int s = s_lo; s <= s_hi; ++s) M = fmaxf(M, ws_ml[(base + s) * 2]);
-    float L = 0.f;
-    for (int s = s_lo; s <= s_hi; ++s) {
+    for (int s = 0; s < ns; ++s) M = fmaxf(M, ws_ml[(base + s) * 2]);
+    for (int s = threadIdx.x; s < ns; s += blockDim.x) {
         const float ms = ws_ml[(base + s) * 2];
-        if (ms > -INFINITY) L += ws_ml[(base + s) * 2 + 1] * expf(ms - M);
+        wgt[s] = (ms > -INFINITY) ? expf(ms - M) : 0.f;
     }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float L = 0.f;
+        for (int s = 0; s < ns; ++s) L += ws_ml[(base + s) * 2 + 1] * wgt[s];
+        inv_l = 1.0f / L;
+    }
+    __syncthreads();
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
         float o = 0.f;
-        for (int s = s_lo; s <= s_hi; ++s) {
-            const float ms = ws_ml[(base + s) * 2];
-            if (ms > -INFINITY) o += ws_o[(base + s) * D + d] * expf(ms - M);
-        }
-        out[(size_t)t * out_stride + (size_t)h * D + d] = tl_from_float<bf16_t>(o / L);
+#pragma unroll 8
+        for (int s = 0; s < ns; ++s) o += ws_o[(base + s) * D + d] * wgt[s];
+        out[(size_t)t * out_stride + (size_t)h * D + d] = tl_from_float<bf16_t>(o * inv_l);
     }
 }
 
@@ -263,7 +287,8 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     TL_CHECK_ARG(d == 32 || d == 64 || d == 128, "tl_attention_mfma: head size %d is not one of 32, 64, 128", d);
     TL_CHECK_ARG(bs >= 8 && bs % 8 == 0, "tl_attention_mfma: page size %d must be a multiple of 8", bs);
     TL_CHECK_ARG(NT == 1 || NT == 2, "tl_attention_mfma: NT=%d must be 1 or 2", NT);
-    TL_CHECK_ARG(nsplit >= 1 && max_tile_groups >= 1, "tl_attention_mfma: bad split or group count");
+    TL_CHECK_ARG(nsplit >= 1 && nsplit <= AM_MAX_SPLITS && max_tile_groups >= 1,
+                 "tl_attention_mfma: bad split count %d (at most %d) or group count", nsplit, AM_MAX_SPLITS);
     TL_CHECK_ARG(nsplit == 1 || (ws_o && ws_ml && pos && split_blocks >= 1),
                  "tl_attention_mfma: split keys need a workspace, positions and a split length");
     TL_CHECK_ARG(q_stride % 8 == 0 && out_stride % 4 == 0 && q_stride >= nq * d && out_stride >= nq * d,

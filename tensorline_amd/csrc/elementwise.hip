@@ -88,9 +88,90 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const R* __restrict__ 
     }
 }
 
+// The same for H a multiple of 4 and at most 16384: one pass, 16-byte accesses, the row kept in
+// registers between the sum of squares and the scaling.
+__device__ __forceinline__ float4 tl_load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 tl_load4(const bf16_t* p) {
+    const uint2 u = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                       __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ void tl_store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void tl_store4(bf16_t* p, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)tl_f2bf_bits(v.x) | ((uint32_t)tl_f2bf_bits(v.y) << 16);
+    u.y = (uint32_t)tl_f2bf_bits(v.z) | ((uint32_t)tl_f2bf_bits(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+}
+
+#define NORM_VPT 4   // float4 per thread at most
+template <typename R, typename O, bool HAS_RES, bool HAS_ROWS>
+__global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict__ x, const R* __restrict__ res,
+                                                               const float* __restrict__ w, O* __restrict__ out,
+                                                               const int32_t* __restrict__ rows, int H, float eps) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const size_t src = HAS_ROWS ? (size_t)rows[r] : (size_t)r;
+    float* xr = x + src * H;
+    const R* rr = HAS_RES ? res + src * H : nullptr;
+    O* orow = out + (size_t)r * H;
+    const int n4 = H >> 2;
+    float4 v[NORM_VPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NORM_VPT; ++i) {
+        const int c4 = threadIdx.x + i * blockDim.x;
+        if (c4 < n4) {
+            float4 a = tl_load4(xr + 4 * c4);
+            if (HAS_RES) {
+                const float4 b = tl_load4(rr + 4 * c4);
+                a.x += b.x;
+                a.y += b.y;
+                a.z += b.z;
+                a.w += b.w;
+                if (!HAS_ROWS) tl_store4(xr + 4 * c4, a);
+            }
+            v[i] = a;
+            ss += a.x * a.x;
+            ss += a.y * a.y;
+            ss += a.z * a.z;
+            ss += a.w * a.w;
+        }
+    }
+    ss = tl_block_sum(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+    for (int i = 0; i < NORM_VPT; ++i) {
+        const int c4 = threadIdx.x + i * blockDim.x;
+        if (c4 < n4) {
+            const float4 g = tl_load4(w + 4 * c4);
+            float4 o;
+            o.x = v[i].x * rstd * g.x;
+            o.y = v[i].y * rstd * g.y;
+            o.z = v[i].z * rstd * g.z;
+            o.w = v[i].w * rstd * g.w;
+            tl_store4(orow + 4 * c4, o);
+        }
+    }
+}
+
 template <typename R, typename O>
 static void launch_add_rmsnorm(float* x, const R* res, const float* w, O* out, const int32_t* rows, int n_rows,
                                int H, float eps, hipStream_t stream) {
+    if (H % 4 == 0 && H <= 1024 * 4 * NORM_VPT) {
+        int threads = ((H / 4 + 63) / 64) * 64;
+        if (threads > 1024) threads = 1024;
+        dim3 grid(n_rows), block(threads);
+        if (res && rows)
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, true, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+        else if (res)
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, true, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+        else if (rows)
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, false, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+        else
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, false, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+        return;
+    }
     dim3 grid(n_rows), block(H >= 2048 ? 512 : 256);
     if (res && rows)
         hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, true, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
@@ -126,7 +207,8 @@ extern "C" int tl_add_rmsnorm(float* x, const void* residual, int res_dtype, con
 // qkv: [T, (nq + 2 nkv) * d] as the fused projection leaves it.  Query heads are rotated in place;
 // key heads are rotated and written to k_cache at the token's slot; value heads are copied to
 // v_cache, which is transposed within a page so that the keys of one page are contiguous for each
-// head dim (what the matrix cores want for the P*V product).  Rotate-half layout over the first `rot` dims of a head (reference: fused.py:34-51):
+// head dim (what the matrix cores want for the P*V product).  Rotate-half layout over the first
+// `rot` dims of a head (reference: fused.py:34-51):
 //   out[i]         = a*cos(theta_i) - b*sin(theta_i)       a = x[i], b = x[i + rot/2]
 //   out[i + rot/2] = b*cos(theta_i) + a*sin(theta_i)       theta_i = pos * inv_freq[i]
 // The angle, sine and cosine are float.  A negative slot skips the cache write of that token.
@@ -136,17 +218,19 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
                                   const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   const int32_t* __restrict__ slots, int nq, int nkv, int d, int rot, int write_kv,
                                   int bs) {
+    __shared__ float cs_s[256], sn_s[256];          // one sine and cosine per rotated pair of the token
     const int t = blockIdx.x;
     const int half = rot / 2;
     const float p = (float)pos[t];
     const int slot = write_kv ? slots[t] : -1;
     T* row = qkv + (size_t)t * (nq + 2 * nkv) * d;
     const int nrot = nq + nkv;  // heads that are rotated: q then k
+    for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(p * inv_freq[i], &sn_s[i], &cs_s[i]);
+    __syncthreads();
     // rotated pairs
     for (int idx = threadIdx.x; idx < nrot * half; idx += blockDim.x) {
         const int h = idx / half, i = idx - h * half;
-        float sn, cs;
-        sincosf(p * inv_freq[i], &sn, &cs);
+        const float sn = sn_s[i], cs = cs_s[i];
         T* hp = row + (size_t)h * d;
         const float a = tl_to_float(hp[i]), b = tl_to_float(hp[i + half]);
         const T o1 = tl_from_float<T>(a * cs - b * sn);
@@ -179,6 +263,7 @@ extern "C" int tl_rope_store(void* qkv, int dtype, const int32_t* pos, const flo
                              int write_kv, int bs, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && nq > 0 && nkv >= 0 && d > 0, "tl_rope_store: bad sizes T=%d nq=%d nkv=%d d=%d", T, nq, nkv, d);
     TL_CHECK_ARG(rot >= 0 && rot <= d && rot % 2 == 0, "tl_rope_store: rotary width %d must be even and <= head size %d", rot, d);
+    TL_CHECK_ARG(rot <= 512, "tl_rope_store: rotary width %d is above the supported 512", rot);
     TL_CHECK_ARG(!write_kv || (k_cache && v_cache && slots && bs > 0), "tl_rope_store: cache write asked for without a cache");
     if (T == 0) return 0;
     dim3 grid(T), block(256);
@@ -206,6 +291,26 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
     out[(size_t)t * I + i] = tl_from_float<T>(g / (1.0f + expf(-g)) * u);
 }
 
+// bfloat16 with I a multiple of 8: 16 bytes of gate and of up per thread
+__global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int I) {
+    const int t = blockIdx.y;
+    const int i8 = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i8 * 8 >= I) return;
+    const bf16_t* row = gu + (size_t)t * 2 * I;
+    const uint4 gv = *reinterpret_cast<const uint4*>(row + i8 * 8);
+    const uint4 uv = *reinterpret_cast<const uint4*>(row + I + i8 * 8);
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
+        const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
+        const float o0 = g0 / (1.0f + expf(-g0)) * u0, o1 = g1 / (1.0f + expf(-g1)) * u1;
+        ow[k] = (uint32_t)tl_f2bf_bits(o0) | ((uint32_t)tl_f2bf_bits(o1) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + (size_t)t * I + i8 * 8) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 extern "C" int tl_silu_mul(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && I > 0, "tl_silu_mul: bad sizes T=%d I=%d", T, I);
     TL_CHECK_ARG(T <= 65535 * 64, "tl_silu_mul: too many rows %d", T);
@@ -214,6 +319,11 @@ extern "C" int tl_silu_mul(const void* gu, void* out, int dtype, int T, int I, h
     for (int t0 = 0; t0 < T; t0 += 65535) {
         const int tn = (T - t0 < 65535) ? T - t0 : 65535;
         dim3 grid(tl_ceil_div(I, 256), tn), block(256);
+        if (dtype == TL_BF16 && I % 8 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+            hipLaunchKernelGGL(silu_mul_bf16x8_kernel, dim3(tl_ceil_div(I / 8, 256), tn), block, 0, stream,
+                               (const bf16_t*)gu + (size_t)t0 * 2 * I, (bf16_t*)out + (size_t)t0 * I, I);
+            continue;
+        }
         if (dtype == TL_F32)
             hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu + (size_t)t0 * 2 * I,
                                (float*)out + (size_t)t0 * I, I);
