@@ -1,0 +1,178 @@
+"""The cache manager on host data: pages per group, tables, windows, state slots, prefix sharing.
+No page is lost, held twice or freed twice, under random orders of requests."""
+import random
+
+import pytest
+import torch
+from hypothesis import given, settings, strategies as st
+
+from tensorline_amd.cache.allocator import BlockAllocator, block_hash
+from tensorline_amd.cache.manager import CacheManager
+from tensorline_amd.parts.spec import CacheNeed, ScheduleEntry, StateNeed
+
+
+def test_allocator_refcount_lru_and_eviction():
+    # the sequence of the reference's own test (tests/test_prefix_cache.py:8-22)
+    a = BlockAllocator(4)
+    x = a.allocate(2)
+    h0 = block_hash(None, [1, 2])
+    a.register(x[0], h0)
+    a.free(x)
+    assert a.num_free == 4 and a.num_cached == 1          # freed but still cached
+    assert a.lookup(h0) == x[0] and a.num_free == 3       # revived from the free list
+    assert a.lookup(h0) == x[0]                           # shared: two references
+    a.free([x[0]])
+    assert a.num_free == 3                                # still referenced once
+    a.free([x[0]])
+    assert a.num_free == 4
+    a.allocate(4)                                         # memory pressure evicts it
+    assert a.num_cached == 0 and a.lookup(h0) is None
+
+
+def test_allocator_details():
+    assert block_hash(block_hash(None, [1]), [2]) != block_hash(block_hash(None, [9]), [2])   # chained over the prefix
+    a = BlockAllocator(3)
+    assert a.allocate(4) is None and a.num_free == 3      # all or nothing
+    x = a.allocate(3)
+    a.free([x[1]])
+    with pytest.raises(AssertionError, match="double free"):
+        a.free([x[1]])
+    a.free([x[0], x[2]])                                  # reversed: the tail page is handed out first
+    assert a.allocate(1) == [x[1]] and a.allocate(1) == [x[2]]
+    b = BlockAllocator(2)
+    y = b.allocate(1)
+    b.register(y[0], 5, content=(None, (1, 2)))
+    assert b.lookup(5, content=(None, (9, 9))) is None    # same hash, other tokens: no hit
+    assert b.lookup(5, content=(None, (1, 2))) == y[0]
+    b.check({y[0]: 2})
+
+
+def manager(needs, schedule=None, states=None, **kw):
+    schedule = schedule or [ScheduleEntry(i) for i in range(len(needs))]
+    states = states or [None] * len(needs)
+    args = dict(page_size=4, num_blocks=16, max_requests=4, dtype=torch.float32, device="cpu")
+    args.update(kw)
+    return CacheManager(needs, schedule, states, **args)
+
+
+def test_groups_tables_and_storage():
+    full, win = CacheNeed(2, 8), CacheNeed(2, 8, window=6)
+    m = manager([full, win, full, None], states=[None, None, None, StateNeed((5,))])
+    assert len(m.groups) == 2 and m.group_of_entry == [0, 1, 0, None]
+    assert m.groups[0].entries == [0, 2] and m.groups[1].entries == [1]
+    k, v = m.storage(2)
+    assert tuple(k.shape) == (17, 4, 2, 8) and tuple(v.shape) == (17, 2, 8, 4)     # one scratch page; V transposed
+    assert m.storage(3) == (None, None) and tuple(m.state[3].shape) == (5, 5)
+    per_page = CacheManager.bytes_per_page([full, win, full, None], [ScheduleEntry(i) for i in range(4)], 4, 2)
+    assert per_page == 3 * 2 * 4 * 2 * 8 * 2
+    assert m.add_request("a") is not None
+    assert m.grow("a", 9) and m.table("a", 0) == m.table("a", 0)[:3] and len(m.table("a", 1)) == 3
+    assert m.num_free(0) == 13 and m.num_free(1) == 13
+    assert m.grow("a", 9) and m.num_free(0) == 13                                  # nothing more to take
+    m.check()
+    m.release("a")
+    assert m.all_free()
+
+
+def test_window_pages_are_given_back_and_used_again():
+    m = manager([CacheNeed(1, 8), CacheNeed(1, 8, window=6)], num_blocks=6)
+    m.add_request("a")
+    computed = 0
+    for n in (5, 4, 3, 7, 1, 1, 1):
+        assert m.grow("a", computed + n)
+        computed += n
+        m.trim("a", computed)
+        m.check()
+        tab = m.table("a", 1)
+        first_needed = computed - 6 + 1
+        for lp, blk in enumerate(tab):
+            assert (blk == -1) == ((lp + 1) * 4 <= first_needed), (lp, computed)    # exactly the pages the window passed
+        assert all(b >= 0 for b in m.table("a", 0))                                 # the full group keeps everything
+    assert computed == 22 and len(m.table("a", 0)) == 6
+    assert m.num_free(1) >= 3            # 22 tokens in 6 pages of 4: the windowed group never holds more than 3 at rest
+    assert m.can_ever_hold(200, step_tokens=4) is False and manager([CacheNeed(1, 8, window=6)], num_blocks=6).can_ever_hold(200, 4)
+    m.release("a")
+    assert m.all_free()
+
+
+def test_shared_cache_entry_and_bad_schedules():
+    need = CacheNeed(2, 8)
+    m = manager([need, need], schedule=[ScheduleEntry(0), ScheduleEntry(0, cache_from=0)])
+    assert m.group_of_entry == [0, 0] and m.storage(1)[0] is m.storage(0)[0] and not m.owns_storage(1)
+    with pytest.raises(ValueError, match="another shape"):
+        manager([need, CacheNeed(1, 8)], schedule=[ScheduleEntry(0), ScheduleEntry(0, cache_from=0)])
+    with pytest.raises(ValueError, match="further back"):
+        manager([CacheNeed(2, 8, window=4), need], schedule=[ScheduleEntry(0), ScheduleEntry(0, cache_from=0)])
+
+
+def test_state_slots():
+    m = manager([None], states=[StateNeed((3,))], max_requests=2)
+    s0, s1 = m.add_request("a"), m.add_request("b")
+    assert {s0, s1} == {0, 1} and m.add_request("c") is None and m.scratch_slot == 2
+    m.state[0][s0].fill_(7.0)
+    m.release("a")
+    assert m.add_request("c") == s0 and torch.all(m.state[0][s0] == 0)              # handed out again from zero
+    with pytest.raises(KeyError):
+        m.add_request("c")
+    m.check()
+
+
+def test_prefix_sharing_through_the_manager():
+    m = manager([CacheNeed(1, 8)], prefix_caching=True)
+    toks = list(range(11))
+    m.add_request("a")
+    assert m.match_prefix("a", toks) == 0 and m.grow("a", 11)
+    m.publish("a", toks, 11)                                                        # two full pages are published
+    m.add_request("b")
+    assert m.match_prefix("b", toks[:8] + [99, 98]) == 8
+    assert m.table("b")[:2] == m.table("a")[:2]
+    m.check()
+    m.add_request("c")
+    assert m.match_prefix("c", toks[:8]) == 4                                       # fully cached: the last page is recomputed
+    m.release("a"); m.release("b"); m.release("c")
+    assert m.all_free() and m.groups[0].allocator.num_cached == 2                   # free, and still there for the next request
+    m.add_request("d")
+    assert m.match_prefix("d", toks) == 8
+    m.release("d")
+    # windows or state switch it off
+    assert not manager([CacheNeed(1, 8, window=4)], prefix_caching=True).prefix_caching
+    assert not manager([CacheNeed(1, 8), None], states=[None, StateNeed((2,))], prefix_caching=True).prefix_caching
+
+
+@settings(max_examples=60, deadline=None)
+@given(seed=st.integers(0, 10 ** 6), window=st.sampled_from([0, 5, 9]), prefix=st.booleans())
+def test_random_orders_keep_every_page_accounted_for(seed, window, prefix):
+    rng = random.Random(seed)
+    needs = [CacheNeed(1, 8), CacheNeed(1, 8, window=window)] if window else [CacheNeed(1, 8)]
+    m = manager(needs, num_blocks=12, max_requests=3, prefix_caching=prefix, allocate_storage=False)
+    live: dict[int, int] = {}
+    toks = {}
+    next_id = 0
+    for _ in range(80):
+        op = rng.random()
+        if op < 0.25 and len(live) < 3:
+            assert m.add_request(next_id) is not None
+            toks[next_id] = [rng.randrange(3) for _ in range(40)]
+            live[next_id] = m.match_prefix(next_id, toks[next_id][:rng.randrange(1, 30)])
+            next_id += 1
+        elif op < 0.8 and live:
+            rid = rng.choice(list(live))
+            n = rng.randrange(1, 9)
+            before = [list(m.table(rid, g)) for g in range(len(m.groups))]
+            free_before = [m.num_free(g) for g in range(len(m.groups))]
+            if live[rid] + n <= 40 and m.grow(rid, live[rid] + n):
+                live[rid] += n
+                m.publish(rid, toks[rid], live[rid])
+                m.trim(rid, live[rid])
+            else:                                               # a failed grow changes nothing
+                assert [list(m.table(rid, g)) for g in range(len(m.groups))] == before
+                assert [m.num_free(g) for g in range(len(m.groups))] == free_before
+        elif live:
+            rid = rng.choice(list(live))
+            m.release(rid)
+            del live[rid]
+        m.check()
+    for rid in list(live):
+        m.release(rid)
+    m.check()
+    assert m.all_free()

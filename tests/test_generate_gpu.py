@@ -245,3 +245,22 @@ def test_toy_mixer_with_state_registers_and_steps(tmp_path):
     c2.grow("again", len(toks))
     again = r2.step([StepEntry("again", toks, 0, list(range(len(toks))))])
     torch.testing.assert_close(again, whole, atol=1e-5, rtol=1e-4)
+
+
+def test_command_line_generate(folder_b, greedy_want):
+    import json
+    import os
+    import subprocess
+    import sys
+    d, w, cfg = folder_b
+    prompts, want = greedy_want
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = [sys.executable, os.path.join(root, "bin", "tensorline"), "generate", "--model", d, "--dtype", "float32",
+           "--num-blocks", "64", "--block-size", "8", "--max-tokens", "24", "--stop-token-id", "-1"]
+    for p in prompts[1:3]:
+        cmd += ["--prompt-ids", " ".join(map(str, p))]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    recs = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")]
+    assert [r["token_ids"] for r in recs] == want[1:3]
+    assert all(r["finish_reason"] == "length" and r["completion_tokens"] == 24 for r in recs)
