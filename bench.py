@@ -74,14 +74,20 @@ def sync():
 
 
 def bench_decode(llm, batch: int, context: int, steps: int, warmup: int, seed: int) -> dict:
-    """Fill ``batch`` sequences so that the last timed step runs at ``context`` tokens, then time
-    ``steps`` decode steps of the whole batch."""
+    """Fill ``batch`` sequences, then time ``steps`` decode steps in which every sequence decodes one
+    token.  Prompts are prefilled in portions under the engine's token budget; sequences admitted
+    early decode while the later ones are still being prefilled (continuous batching), so prompts
+    are shortened by the number of prefill steps: no sequence passes ``context`` tokens before the
+    last timed step, and none finishes before it."""
     from tensorline_amd import SamplingParams
     cfg = llm.model_config
-    prompt_len = context - (warmup + steps)
-    assert prompt_len >= 1
     eng = llm.engine
-    reqs = [eng.add_request(p, SamplingParams(max_tokens=warmup + steps + 8, stop_token_ids={-1}))
+    budget = eng.scheduler.max_batched_tokens
+    prompt_len = context - (warmup + steps) - 1
+    prefill_steps = -(-batch * prompt_len // budget) + 1
+    prompt_len -= prefill_steps if batch > 1 else 0
+    assert prompt_len >= 1
+    reqs = [eng.add_request(p, SamplingParams(max_tokens=10 ** 9, stop_token_ids={-1}))
             for p in random_prompts(batch, prompt_len, cfg.vocab_size, seed)]
     t0 = time.perf_counter()
     while any(r.num_computed < r.prompt_len for r in reqs):          # prefill, in portions
@@ -91,15 +97,22 @@ def bench_decode(llm, batch: int, context: int, steps: int, warmup: int, seed: i
     for _ in range(warmup):
         eng.step()
     sync()
-    replays0 = eng.counters()["graph_replays"]
+    assert all(not r.done for r in reqs) and len(eng.scheduler.running) == batch and not eng.scheduler.waiting
+    c0 = eng.counters()
+    lens0 = [len(r.tokens) for r in reqs]
     t0 = time.perf_counter()
     for _ in range(steps):
         eng.step()
     sync()
     dt = time.perf_counter() - t0
-    assert all(r.num_generated >= warmup + steps for r in reqs), "a decode step did not advance every sequence"
-    out = {"tok_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3, "fill_s": fill_s,
-           "graph_replays": eng.counters()["graph_replays"] - replays0}
+    c1 = eng.counters()
+    lens1 = [len(r.tokens) for r in reqs]
+    assert c1["tokens_generated"] - c0["tokens_generated"] == batch * steps, "a timed step did not decode every sequence"
+    assert all(b - a == steps for a, b in zip(lens0, lens1)) and max(lens1) <= context + 1
+    assert c1["preemptions"] == c0["preemptions"], "a sequence was preempted inside the timed steps"
+    mean_ctx = (sum(lens0) + sum(lens1)) / (2.0 * batch)
+    out = {"tok_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3, "fill_s": fill_s, "mean_context": mean_ctx,
+           "graph_replays": c1["graph_replays"] - c0["graph_replays"]}
     for r in reqs:
         eng.abort(r)
     assert llm.cache.all_free()
@@ -169,8 +182,7 @@ def main() -> int:
             points[f"decode_b{b}"] = round(bench_decode(llm, b, args.context, k, 4, args.seed + 3 + b)["tok_s"], 1)
 
     step_s = main_run["ms_per_step"] / 1e3
-    mean_ctx = args.context - args.steps / 2.0
-    achieved = decode_bytes(cfg, args.batch, int(mean_ctx), elem) / step_s / 1e9
+    achieved = decode_bytes(cfg, args.batch, int(main_run["mean_context"]), elem) / step_s / 1e9
     flops = prefill_flops(cfg, args.prefill_tokens)
     line = {
         "metric": "decode tok/s @ batch 8, context 4096 (Qwen2.5-7B shape)",
@@ -192,7 +204,7 @@ def main() -> int:
             "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "page_size": page,
             "prefill_tokens": args.prefill_tokens, "graphs": not args.no_graphs, "sampling": "greedy",
-            "decode_graph_replays": main_run["graph_replays"],
+            "decode_graph_replays": main_run["graph_replays"], "mean_context": round(main_run["mean_context"], 1),
         },
         "prefill": {"value": round(pre["tok_s"], 1), "tokens": args.prefill_tokens, "ms": round(pre["s"] * 1e3, 3),
                     "frac": round(flops / pre["s"] / PEAK_FLOPS[dtype_key], 4)},

@@ -62,10 +62,62 @@ __global__ __launch_bounds__(SM_THREADS) void argmax_kernel(const float* __restr
     if (threadIdx.x == 0) out[r] = best;
 }
 
-extern "C" int tl_argmax(const float* logits, int ld, int R, int V, int32_t* out, hipStream_t stream) {
+// Wide rows are cut into chunks so that a few rows still fill the GPU: one work-group per (row,
+// chunk) finds the chunk's best, a second kernel the row's best among them.  Ties go to the lower
+// index in both steps, so the answer is that of the one-kernel form.
+__global__ __launch_bounds__(256) void argmax_chunk_kernel(const float* __restrict__ logits, int ld, int V,
+                                                                  int chunk, float* __restrict__ pval,
+                                                                  int32_t* __restrict__ pidx) {
+    __shared__ ArgMax sh[16];
+    const int r = blockIdx.x, ch = blockIdx.y;
+    const int c0 = ch * chunk;
+    const int n = (V - c0 < chunk) ? V - c0 : chunk;
+    const float* row = logits + (size_t)r * ld + c0;
+    const int best = block_argmax(row, n, sh);
+    if (threadIdx.x == 0) {
+        pval[(size_t)r * gridDim.y + ch] = row[best];
+        pidx[(size_t)r * gridDim.y + ch] = c0 + best;
+    }
+}
+
+__global__ void argmax_final_kernel(const float* __restrict__ pval, const int32_t* __restrict__ pidx, int nch,
+                                    int32_t* __restrict__ out) {
+    const int r = blockIdx.x;
+    ArgMax best;
+    best.v = -INFINITY;
+    best.i = 0x7fffffff;
+    for (int c = threadIdx.x; c < nch; c += TL_WAVE) {
+        ArgMax cur;
+        cur.v = pval[(size_t)r * nch + c];
+        cur.i = pidx[(size_t)r * nch + c];
+        best = argmax_better(best, cur);
+    }
+#pragma unroll
+    for (int off = TL_WAVE / 2; off > 0; off >>= 1) {
+        ArgMax o;
+        o.v = __shfl_xor(best.v, off, TL_WAVE);
+        o.i = __shfl_xor(best.i, off, TL_WAVE);
+        best = argmax_better(best, o);
+    }
+    if (threadIdx.x == 0) out[r] = (best.i == 0x7fffffff) ? 0 : best.i;
+}
+
+#define AM_CHUNKS 64
+// scratch: room for R * 64 floats and R * 64 int32 when V > 8192 (may be null otherwise)
+extern "C" int tl_argmax(const float* logits, int ld, int R, int V, int32_t* out, float* scratch_val,
+                         int32_t* scratch_idx, hipStream_t stream) {
     TL_CHECK_ARG(R >= 0 && V > 0 && ld >= V, "tl_argmax: bad sizes R=%d V=%d ld=%d", R, V, ld);
     if (R == 0) return 0;
-    hipLaunchKernelGGL(argmax_kernel, dim3(R), dim3(SM_THREADS), 0, stream, logits, ld, V, out);
+    if (V <= 8192 || !scratch_val || !scratch_idx || R > 65535) {
+        hipLaunchKernelGGL(argmax_kernel, dim3(R), dim3(SM_THREADS), 0, stream, logits, ld, V, out);
+        TL_CHECK_LAUNCH("tl_argmax");
+        return 0;
+    }
+    const int chunk = tl_ceil_div(V, AM_CHUNKS);
+    const int nch = tl_ceil_div(V, chunk);
+    hipLaunchKernelGGL(argmax_chunk_kernel, dim3(R, nch), dim3(256), 0, stream, logits, ld, V, chunk, scratch_val,
+                       scratch_idx);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(R), dim3(TL_WAVE), 0, stream, scratch_val, scratch_idx, nch, out);
     TL_CHECK_LAUNCH("tl_argmax");
     return 0;
 }

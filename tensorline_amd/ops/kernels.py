@@ -384,7 +384,11 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
     if out is None:
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
     _i32(out, "argmax output", R)
-    _call("tl_argmax", _ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(out), _stream())
+    sv = si = None
+    if V > 8192:            # wide rows: per-chunk bests, then the row's best among them
+        sv = torch.empty(R * 64, dtype=torch.float32, device=logits.device)
+        si = torch.empty(R * 64, dtype=torch.int32, device=logits.device)
+    _call("tl_argmax", _ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(out), _ptr(sv), _ptr(si), _stream())
     return out
 
 
