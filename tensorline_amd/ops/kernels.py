@@ -190,7 +190,7 @@ def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     return _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled)
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 16     # the streaming kernel serves up to 64 rows; above 16 the library is faster today
 
 
 def _skinny_ok(a: torch.Tensor, shuffled: torch.Tensor | None, M: int, K: int, lda: int) -> bool:
