@@ -17,13 +17,35 @@
 // the k values of unit 4*chunk + g.  No barrier is needed for that: a wave's LDS operations
 // complete in order.  The accumulator of lane l, register i, is C[m = l % 16][n = 4*(l / 16) + i].
 //
-// DUAL: the work-group owns tile t of the first I/16 tiles and tile t of the next I/16 and writes
-// silu(first) * second, the SwiGLU gate, for a fused [2I, K] gate/up matrix.
+// Two tiles per work-group (MODE_SWIGLU, MODE_QKV), sharing the A fragments:
+//  * MODE_SWIGLU owns tile t of the first I/16 tiles and tile t of the next I/16 of a fused
+//    [2I, K] gate/up matrix and writes silu(first) * second.
+//  * MODE_QKV owns, in head h of a fused q/k/v projection, tiles j and j + d/32: the two halves
+//    that rotate-half RoPE pairs.  Its epilogue adds the bias, rotates query and key heads by the
+//    token's position (angle pos * inv_freq[i] in float, as tl_rope_store does), writes queries to
+//    a [M, nq*d] matrix and keys and values straight into the paged cache at the token's slot:
+//    the projection, the position encoding and the cache write of a decode step in one kernel.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+#define MODE_PLAIN 0
+#define MODE_SWIGLU 1
+#define MODE_QKV 2
+
+// what MODE_QKV needs beyond the product
+struct QkvArgs {
+    const int32_t* pos;        // [M] positions
+    const float* inv_freq;     // [d/2]
+    const int32_t* slots;      // [M] cache rows (negative: do not store)
+    bf16_t* q_out;             // [M, nq*d]
+    bf16_t* k_cache;           // [pages, page, nkv, d]
+    bf16_t* v_cache;           // [pages, nkv, d, page]
+    int nq, nkv, d, bs;
+};
+
+#define SK_MAX_LDS (80 * 1024)          // LDS of a work-group; a CU has 160 KB
 #define SK_SC 128                    // k values staged per step (4 chunks of 32)
 #define SK_UNITS (SK_SC / 8)         // 16-byte units per row of a step
 #define SK_ROWPAD 17                 // rows per unit in LDS: 16 + 1 of padding
@@ -38,18 +60,25 @@ __device__ __forceinline__ void wave_lds_order() {
     asm volatile("" ::: "memory");
 }
 
-template <int MT, bool DUAL, typename TO>
-__global__ __launch_bounds__(DUAL ? 256 : 1024) void gemm_skinny_kernel(
+template <int MT, int MODE, typename TO>
+__global__ __launch_bounds__(MODE == MODE_SWIGLU ? 256 : 1024) void gemm_skinny_kernel(
     const bf16_t* __restrict__ A, const uint4* __restrict__ Ws, const float* __restrict__ bias, TO* __restrict__ C,
-    int M, int n_out, int K, int K32, int lda, int ldc, int second_tile) {
+    int M, int n_out, int K, int K32, int lda, int ldc, int second_tile, QkvArgs qa) {
     extern __shared__ uint4 smem[];
+    constexpr bool DUAL = MODE != MODE_PLAIN;
     constexpr int NACC = MT * (DUAL ? 2 : 1);
     constexpr int XS_PER_WAVE = MT * SK_UNITS * SK_ROWPAD;     // in uint4
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int r = lane & 15, g = lane >> 4;
-    const int tile = blockIdx.x;
+    int tile = blockIdx.x, tile2 = second_tile + blockIdx.x;
+    if (MODE == MODE_QKV) {
+        const int pph = qa.d / 32;                   // tile pairs per head
+        const int head = blockIdx.x / pph, j = blockIdx.x - head * pph;
+        tile = head * (qa.d / 16) + j;
+        tile2 = tile + pph;
+    }
     const uint4* w1 = Ws + (size_t)tile * K32 * 64 + lane;
-    const uint4* w2 = DUAL ? Ws + (size_t)(second_tile + tile) * K32 * 64 + lane : nullptr;
+    const uint4* w2 = DUAL ? Ws + (size_t)tile2 * K32 * 64 + lane : nullptr;
     uint4* xs = smem + (size_t)wave * XS_PER_WAVE;
     const uint4 zero = make_uint4(0, 0, 0, 0);
 
@@ -161,7 +190,37 @@ __global__ __launch_bounds__(DUAL ? 256 : 1024) void gemm_skinny_kernel(
             v += red[((size_t)w * NACC * 4 + mt * 4 + i) * 64 + l];
             if (DUAL) u += red[((size_t)w * NACC * 4 + (MT + mt) * 4 + i) * 64 + l];
         }
-        if (DUAL) {
+        if (MODE == MODE_QKV) {
+            // v, u: dims idx and idx + d/2 of head `head` for token m
+            const int d = qa.d, half = d / 2;
+            const int head = n / d, idx = n - head * d;
+            if (bias) {
+                v += bias[n];
+                u += bias[n + half];
+            }
+            const int slot = qa.slots[m];
+            if (head < qa.nq + qa.nkv) {
+                float sn, cs;
+                sincosf((float)qa.pos[m] * qa.inv_freq[idx], &sn, &cs);
+                const float o1 = v * cs - u * sn, o2 = u * cs + v * sn;
+                if (head < qa.nq) {
+                    bf16_t* qp = qa.q_out + (size_t)m * qa.nq * d + (size_t)head * d + idx;
+                    qp[0] = tl_from_float<bf16_t>(o1);
+                    qp[half] = tl_from_float<bf16_t>(o2);
+                } else if (slot >= 0) {
+                    bf16_t* kp = qa.k_cache + ((size_t)slot * qa.nkv + (head - qa.nq)) * d + idx;
+                    kp[0] = tl_from_float<bf16_t>(o1);
+                    kp[half] = tl_from_float<bf16_t>(o2);
+                }
+            } else if (slot >= 0) {
+                const int page = slot / qa.bs, off = slot - page * qa.bs;
+                bf16_t* vp = qa.v_cache + (((size_t)page * qa.nkv + (head - qa.nq - qa.nkv)) * d + idx) * qa.bs + off;
+                vp[0] = tl_from_float<bf16_t>(v);
+                vp[(size_t)half * qa.bs] = tl_from_float<bf16_t>(u);
+            }
+            continue;
+        }
+        if (MODE == MODE_SWIGLU) {
             v = v / (1.0f + expf(-v)) * u;
         } else if (bias) {
             v += bias[n];
@@ -180,22 +239,23 @@ static int pick_waves(int tiles, int nsc, int MT, int nacc, int max_waves) {
     // enough waves in flight to cover HBM latency on 256 CUs; K is split among the waves of a group
     int w = 1;
     while (w < max_waves && tiles * w < 4096 && nsc >= 2 * w) w <<= 1;
-    while (w > 1 && (size_t)w * lds_per_wave(MT, nacc) > 64 * 1024) w >>= 1;
+    while (w > 1 && (size_t)w * lds_per_wave(MT, nacc) > SK_MAX_LDS) w >>= 1;
     return w;
 }
 
-template <int MT, bool DUAL, typename TO>
+template <int MT, int MODE, typename TO>
 static void launch_skinny(const bf16_t* A, const uint4* Ws, const float* bias, TO* C, int M, int n_out, int K, int K32,
-                          int lda, int ldc, int second_tile, hipStream_t stream) {
-    const int tiles = tl_ceil_div(n_out, 16);
-    const int nacc = MT * (DUAL ? 2 : 1);
-    const int nwaves = pick_waves(tiles, (K32 + 3) / 4, MT, nacc, DUAL ? 4 : 16);
+                          int lda, int ldc, int second_tile, hipStream_t stream, QkvArgs qa = QkvArgs()) {
+    // the grid: one group per tile, or per pair of tiles in the two-tile modes
+    const int groups = (MODE == MODE_QKV) ? tl_ceil_div(n_out, 32) : tl_ceil_div(n_out, 16);
+    const int nacc = MT * (MODE != MODE_PLAIN ? 2 : 1);
+    const int nwaves = pick_waves(groups, (K32 + 3) / 4, MT, nacc, MODE == MODE_SWIGLU ? 4 : 16);
     const size_t smem = (size_t)nwaves * lds_per_wave(MT, nacc);
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, DUAL, TO>), dim3(tiles), dim3(nwaves * 64), smem, stream, A, Ws, bias, C,
-                       M, n_out, K, K32, lda, ldc, second_tile);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, MODE, TO>), dim3(groups), dim3(nwaves * 64), smem, stream, A, Ws, bias, C,
+                       M, n_out, K, K32, lda, ldc, second_tile, qa);
 }
 
-template <bool DUAL, typename TO>
+template <int DUAL, typename TO>
 static int dispatch_skinny(const bf16_t* A, const uint4* Ws, const float* bias, TO* C, int M, int n_out, int K, int K32,
                            int lda, int ldc, int second_tile, hipStream_t stream) {
     // Row counts are served in classes of 16, 32 and 64 rows, the sizes decode batches are padded
@@ -225,9 +285,9 @@ extern "C" int tl_gemm_skinny(const void* A, const void* Ws, const float* bias, 
     if (M == 0) return 0;
     const int K32 = tl_ceil_div(K, 32);
     if (c_dtype == TL_F32)
-        return dispatch_skinny<false, float>((const bf16_t*)A, (const uint4*)Ws, bias, (float*)C, M, N, K, K32, lda, ldc, 0, stream);
+        return dispatch_skinny<MODE_PLAIN, float>((const bf16_t*)A, (const uint4*)Ws, bias, (float*)C, M, N, K, K32, lda, ldc, 0, stream);
     if (c_dtype == TL_BF16)
-        return dispatch_skinny<false, bf16_t>((const bf16_t*)A, (const uint4*)Ws, bias, (bf16_t*)C, M, N, K, K32, lda, ldc, 0, stream);
+        return dispatch_skinny<MODE_PLAIN, bf16_t>((const bf16_t*)A, (const uint4*)Ws, bias, (bf16_t*)C, M, N, K, K32, lda, ldc, 0, stream);
     return tl_fail("tl_gemm_skinny: unknown output dtype %d", c_dtype);
 }
 
@@ -239,6 +299,37 @@ extern "C" int tl_gemm_skinny_swiglu(const void* A, const void* Ws, void* C, int
     TL_CHECK_ARG(I % 16 == 0, "tl_gemm_skinny_swiglu: I=%d must be a multiple of 16", I);
     TL_CHECK_ARG(ldc >= I, "tl_gemm_skinny_swiglu: output row stride %d < I=%d", ldc, I);
     if (M == 0) return 0;
-    return dispatch_skinny<true, bf16_t>((const bf16_t*)A, (const uint4*)Ws, nullptr, (bf16_t*)C, M, I, K,
+    return dispatch_skinny<MODE_SWIGLU, bf16_t>((const bf16_t*)A, (const uint4*)Ws, nullptr, (bf16_t*)C, M, I, K,
                                          tl_ceil_div(K, 32), lda, ldc, I / 16, stream);
+}
+
+// The fused q/k/v projection of a decode step: Ws is the shuffled copy of the [(nq + 2 nkv) d, K]
+// matrix, bias float [(nq + 2 nkv) d] or null.  Writes rotated queries to q_out [M, nq*d] and rotated
+// keys and the values into the cache at slots[m] (k_cache [pages, page, nkv, d], v_cache
+// [pages, nkv, d, page]).  Full-width rotate-half RoPE only: inv_freq holds d/2 values.
+extern "C" int tl_gemm_skinny_qkv_rope(const void* A, const void* Ws, const float* bias, const int32_t* pos,
+                                       const float* inv_freq, const int32_t* slots, void* q_out, void* k_cache,
+                                       void* v_cache, int M, int K, int lda, int nq, int nkv, int d, int bs,
+                                       hipStream_t stream) {
+    const int N = (nq + 2 * nkv) * d;
+    if (int rc = check_skinny(A, Ws, q_out, M, N, K, lda, 1)) return rc;
+    TL_CHECK_ARG(M <= 16, "tl_gemm_skinny_qkv_rope: M=%d is above 16", M);
+    TL_CHECK_ARG(d % 32 == 0 && d > 0 && nq > 0 && nkv > 0 && bs > 0, "tl_gemm_skinny_qkv_rope: bad sizes d=%d nq=%d nkv=%d page=%d", d, nq, nkv, bs);
+    TL_CHECK_ARG(pos && inv_freq && slots && k_cache && v_cache, "tl_gemm_skinny_qkv_rope: missing argument");
+    if (M == 0) return 0;
+    QkvArgs qa;
+    qa.pos = pos;
+    qa.inv_freq = inv_freq;
+    qa.slots = slots;
+    qa.q_out = (bf16_t*)q_out;
+    qa.k_cache = (bf16_t*)k_cache;
+    qa.v_cache = (bf16_t*)v_cache;
+    qa.nq = nq;
+    qa.nkv = nkv;
+    qa.d = d;
+    qa.bs = bs;
+    launch_skinny<1, MODE_QKV, bf16_t>((const bf16_t*)A, (const uint4*)Ws, bias, (bf16_t*)nullptr, M, N, K,
+                                       tl_ceil_div(K, 32), lda, N, 0, stream, qa);
+    TL_CHECK_LAUNCH("tl_gemm_skinny_qkv_rope");
+    return 0;
 }

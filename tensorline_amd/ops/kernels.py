@@ -264,6 +264,34 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, who: str) -> 
            f"{who}: value cache must be contiguous [pages, nkv, d, page] matching the key cache")
 
 
+def qkv_rope_store(h: torch.Tensor, shuffled: torch.Tensor, bias: torch.Tensor | None, pos: torch.Tensor,
+                   inv_freq: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                   k_cache: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor) -> torch.Tensor | None:
+    """The projection, position encoding and cache write of a decode step in one kernel: returns the
+    rotated queries [M, nq*d]; rotated keys and the values go into the cache at ``slots``.  Returns
+    None when the kernel does not take the case (then the three separate kernels run): it needs
+    bfloat16, at most 16 rows, a head size that is a multiple of 32 and full-width rotation."""
+    M, K = h.shape
+    N = (num_heads + 2 * num_kv_heads) * head_dim
+    if not (h.dtype == torch.bfloat16 and shuffled is not None and M <= 16 and head_dim % 32 == 0
+            and inv_freq is not None and 2 * inv_freq.numel() == head_dim and h.stride(1) == 1
+            and K % 8 == 0 and h.data_ptr() % 16 == 0 and (M == 1 or h.stride(0) % 8 == 0)):
+        return None
+    _on_gpu(h, shuffled, bias, pos, inv_freq, k_cache, v_cache, slots)
+    _check_shuffled(shuffled, N, K)
+    _check_caches(k_cache, v_cache, h.dtype, num_kv_heads, head_dim, "qkv_rope_store")
+    _i32(pos, "pos", M)
+    _i32(slots, "slots", M)
+    _check(inv_freq.dtype == torch.float32 and inv_freq.is_contiguous(), "qkv_rope_store: inv_freq must be float32")
+    if bias is not None:
+        _check(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == N, "qkv_rope_store: bad bias")
+    q = torch.empty(M, num_heads * head_dim, dtype=h.dtype, device=h.device)
+    _call("tl_gemm_skinny_qkv_rope", _ptr(h), _ptr(shuffled), _ptr(bias), _ptr(pos), _ptr(inv_freq), _ptr(slots),
+          _ptr(q), _ptr(k_cache), _ptr(v_cache), M, K, h.stride(0) if M > 1 else K, num_heads, num_kv_heads,
+          head_dim, k_cache.shape[1], _stream())
+    return q
+
+
 def rope_store(qkv: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor | None, num_heads: int,
                num_kv_heads: int, head_dim: int, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None,
                slots: torch.Tensor | None) -> None:

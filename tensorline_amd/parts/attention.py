@@ -70,12 +70,17 @@ class PagedAttention(Part):
 
     # ---- one step ------------------------------------------------------------------------
     def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
-        qkv = self.qkv(h)
         nkv_local = self.num_kv_heads if self.kv_proj else 0
         write = cache.write and self.kv_proj
-        self.position.apply_and_store(qkv, ctx.pos, self.num_heads, nkv_local, self.head_dim,
-                                      cache.k if write else None, cache.v if write else None,
-                                      cache.slots if write else None)
+        qkv = None
+        fused = getattr(self.position, "project_rotate_store", None)
+        if fused is not None and write:
+            qkv = fused(h, self.qkv, ctx.pos, self.num_heads, nkv_local, self.head_dim, cache.k, cache.v, cache.slots)
+        if qkv is None:
+            qkv = self.qkv(h)
+            self.position.apply_and_store(qkv, ctx.pos, self.num_heads, nkv_local, self.head_dim,
+                                          cache.k if write else None, cache.v if write else None,
+                                          cache.slots if write else None)
         o = kernels.paged_attention(qkv, cache.k, cache.v, cache.tables, ctx.seq_of_token, ctx.pos,
                                     self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
                                     window=self.window, q_start=ctx.q_start, ctx_start=ctx.ctx_start,

@@ -4,7 +4,9 @@ cache (fused, because the rotated key is what the cache holds; reference: paged.
 
 Interface: ``apply_and_store(qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
 slots)`` rotates the query heads of the fused projection in place and stores keys and values at
-``slots`` (``k_cache`` None: nothing is stored).
+``slots`` (``k_cache`` None: nothing is stored).  A position encoding may also offer
+``project_rotate_store(h, qkv_linear, ...)``, which does the projection as well and returns the
+queries, or None to decline; the attention mixer tries it first.
 """
 from __future__ import annotations
 
@@ -33,6 +35,14 @@ class RotaryEmbedding:
 
     def apply_and_store(self, qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots) -> None:
         kernels.rope_store(qkv, pos, self.inv_freq, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots)
+
+    def project_rotate_store(self, h, qkv_linear, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots):
+        """Optional shortcut for few-row steps: projection, rotation and cache write in one kernel.
+        Returns the rotated queries [T, nq*d], or None when that kernel does not take the case."""
+        if self.rotary_dim != head_dim or k_cache is None:
+            return None
+        return kernels.qkv_rope_store(h, qkv_linear.shuffled, qkv_linear.bias, pos, self.inv_freq, num_heads,
+                                      num_kv_heads, head_dim, k_cache, v_cache, slots)
 
 
 @register_position("none")

@@ -33,6 +33,10 @@ def add_rmsnorm(x, residual, weight, eps, out_dtype, rows=None, out=None):
     return r.to(out_dtype)
 
 
+def qkv_rope_store(*args, **kw):
+    return None
+
+
 def shuffle_weight(weight):
     return None
 
@@ -121,7 +125,7 @@ def sample(logits, temperature, top_p, uniform, out=None):
     return res
 
 
-ALL = ["require_gpu", "embed", "add_rmsnorm", "linear", "rope_store", "paged_attention", "silu_mul", "swiglu_gate_up", "shuffle_weight", "argmax",
+ALL = ["require_gpu", "embed", "add_rmsnorm", "linear", "rope_store", "paged_attention", "silu_mul", "swiglu_gate_up", "shuffle_weight", "qkv_rope_store", "argmax",
        "sample"]
 
 

@@ -159,6 +159,45 @@ def test_rope_store(dtype, nq, nkv, d, rot):
     torch.testing.assert_close(qkv0, keep, atol=0, rtol=0)
 
 
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("nq,nkv,d,Kd", [(6, 2, 32, 192), (28, 4, 128, 3584), (4, 4, 64, 264), (5, 1, 96, 120)])
+def test_fused_projection_rotation_and_cache_write(M, nq, nkv, d, Kd):
+    """One kernel for q/k/v projection + bias + RoPE + cache write against the three separate kernels."""
+    torch.manual_seed(M + nq)
+    bs, pages, theta = 8, 12, 1e6
+    N = (nq + 2 * nkv) * d
+    h = torch.randn(M, Kd, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(torch.bfloat16)
+    b = torch.randn(N, device=DEV)
+    pos = torch.randint(0, 4000, (M,), dtype=torch.int32, device=DEV)
+    slots = torch.randperm(pages * bs, device=DEV)[:M].to(torch.int32)
+    if M > 2:
+        slots[2] = -1
+    inv_freq = (theta ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)).float().to(DEV)
+    mk = lambda: (torch.full((pages, bs, nkv, d), 7.0, device=DEV).to(torch.bfloat16),
+                  torch.full((pages, nkv, d, bs), 7.0, device=DEV).to(torch.bfloat16))
+    kc, vc = mk()
+    q = K().qkv_rope_store(h, K().shuffle_weight(w), b, pos, inv_freq, nq, nkv, d, kc, vc, slots)
+    assert q is not None and tuple(q.shape) == (M, nq * d)
+    # the same from the plain formulas in float64
+    qkv = (h.double() @ w.double().T + b.double()).cpu().view(M, nq + 2 * nkv, d)
+    want_q = plain.rope(qkv[:, :nq], pos.cpu(), theta)
+    want_k = plain.rope(qkv[:, nq:nq + nkv], pos.cpu(), theta)
+    torch.testing.assert_close(q.double().cpu().view(M, nq, d), want_q, atol=3e-2, rtol=3e-2)
+    ok = slots.cpu() >= 0
+    sl = slots.cpu()[ok].long()
+    kf = kc.double().cpu().view(-1, nkv, d)
+    vf = vc.double().cpu().permute(0, 3, 1, 2).reshape(-1, nkv, d)
+    torch.testing.assert_close(kf[sl], want_k[ok], atol=3e-2, rtol=3e-2)
+    torch.testing.assert_close(vf[sl], qkv[:, nq + nkv:][ok], atol=3e-2, rtol=3e-2)
+    untouched = torch.ones(pages * bs, dtype=torch.bool)
+    untouched[sl] = False
+    assert torch.all(kf[untouched] == 7.0) and torch.all(vf[untouched] == 7.0)
+    # cases it declines: float32, too many rows, partial rotation
+    assert K().qkv_rope_store(h.float(), None, b, pos, inv_freq, nq, nkv, d, kc, vc, slots) is None
+    assert K().qkv_rope_store(h, K().shuffle_weight(w), b, pos, inv_freq[: d // 4].contiguous(), nq, nkv, d, kc, vc, slots) is None
+
+
 def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False, path=None, split_keys=None):
     """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries."""
     torch.manual_seed(seed)
