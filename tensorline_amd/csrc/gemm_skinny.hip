@@ -1,4 +1,4 @@
-// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for few rows (M <= 64), bfloat16 inputs: the matrix
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for few rows (M <= 16), bfloat16 inputs: the matrix
 // products of a decode step.  The work is streaming W once from HBM.
 //
 // W is read from a copy laid out for the matrix cores ("shuffled", made once when the weights are
@@ -258,17 +258,14 @@ static void launch_skinny(const bf16_t* A, const uint4* Ws, const float* bias, T
 template <int DUAL, typename TO>
 static int dispatch_skinny(const bf16_t* A, const uint4* Ws, const float* bias, TO* C, int M, int n_out, int K, int K32,
                            int lda, int ldc, int second_tile, hipStream_t stream) {
-    // Row counts are served in classes of 16, 32 and 64 rows, the sizes decode batches are padded
-    // to for graph replay: a batch and its padded twin split K alike and give the same bits.
-    if (M <= 16) launch_skinny<1, DUAL, TO>(A, Ws, bias, C, M, n_out, K, K32, lda, ldc, second_tile, stream);
-    else if (M <= 32) launch_skinny<2, DUAL, TO>(A, Ws, bias, C, M, n_out, K, K32, lda, ldc, second_tile, stream);
-    else launch_skinny<4, DUAL, TO>(A, Ws, bias, C, M, n_out, K, K32, lda, ldc, second_tile, stream);
+    // one 16-row MFMA tile of A; more rows go to gemm_rows64.hip
+    launch_skinny<1, DUAL, TO>(A, Ws, bias, C, M, n_out, K, K32, lda, ldc, second_tile, stream);
     TL_CHECK_LAUNCH("tl_gemm_skinny");
     return 0;
 }
 
 static int check_skinny(const void* A, const void* Ws, const void* C, int M, int N, int K, int lda, int ldc) {
-    TL_CHECK_ARG(M >= 0 && M <= 64, "tl_gemm_skinny: M=%d is outside [0, 64]", M);
+    TL_CHECK_ARG(M >= 0 && M <= 16, "tl_gemm_skinny: M=%d is outside [0, 16]", M);
     TL_CHECK_ARG(N > 0 && K > 0, "tl_gemm_skinny: bad sizes N=%d K=%d", N, K);
     TL_CHECK_ARG(K % 8 == 0 && lda % 8 == 0, "tl_gemm_skinny: K=%d and the row stride %d must be multiples of 8", K, lda);
     TL_CHECK_ARG(((uintptr_t)A % 16) == 0 && ((uintptr_t)Ws % 16) == 0, "tl_gemm_skinny: operands must be 16-byte aligned");

@@ -178,7 +178,8 @@ def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
                f"linear: bias must be float32 of {N} entries")
     out_dtype = out_dtype or a.dtype
     if out is None:
-        if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M > SKINNY_MAX_ROWS:
+        if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and (
+                M > ROWS64_MAX_ROWS or (M > SKINNY_MAX_ROWS and shuffled is None)):
             return _library_linear(a, weight, bias, out_dtype)
         out = torch.empty(M, N, dtype=out_dtype, device=a.device)
     _check(out.dim() == 2 and tuple(out.shape) == (M, N) and out.stride(1) == 1 and out.dtype == out_dtype,
@@ -190,12 +191,27 @@ def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
     return _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled)
 
 
-SKINNY_MAX_ROWS = 16     # the streaming kernel serves up to 64 rows; above 16 the library is faster today
+SKINNY_MAX_ROWS = 16     # rows the few-row kernel serves (one 16-row MFMA tile)
+ROWS64_MAX_ROWS = 64     # rows the 17..64-row kernel serves; above that the library
 
 
 def _skinny_ok(a: torch.Tensor, shuffled: torch.Tensor | None, M: int, K: int, lda: int) -> bool:
     return (shuffled is not None and a.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS
             and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0)
+
+
+def _rows64_ok(a: torch.Tensor, shuffled: torch.Tensor | None, M: int, K: int, lda: int) -> bool:
+    return (shuffled is not None and a.dtype == torch.bfloat16 and SKINNY_MAX_ROWS < M <= ROWS64_MAX_ROWS
+            and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0)
+
+
+def _rows64(a, shuffled, bias, out, M, N, K, lda, ldc, swiglu: bool) -> torch.Tensor:
+    """17 to 64 rows: 128 columns per work-group, rows shared through LDS, K split over the grid."""
+    shares = library().tl_gemm_rows64_shares(M, N, K)
+    ws = torch.empty(shares * M * N, dtype=torch.float32, device=a.device) if shares > 1 else None
+    _call("tl_gemm_rows64", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), _code(out, "linear output"), _ptr(ws),
+          M, N, K, lda, ldc, shares, 1 if swiglu else 0, _stream())
+    return out
 
 
 def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled=None) -> torch.Tensor:
@@ -206,6 +222,8 @@ def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled=None) -> 
         _call("tl_gemm_skinny", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), _code(out, "linear output"),
               M, N, K, lda, ldc, _stream())
         return out
+    if _rows64_ok(a, shuffled, M, K, lda):
+        return _rows64(a, shuffled, bias, out, M, N, K, lda, ldc, swiglu=False)
     _call("tl_gemm_generic", _ptr(a), _code(a, "linear input"), _ptr(weight), _code(weight, "linear weight"),
           _ptr(bias), _ptr(out), _code(out, "linear output"), M, N, K, lda, ldc, _stream())
     return out
@@ -250,6 +268,9 @@ def swiglu_gate_up(h: torch.Tensor, gate_up_weight: torch.Tensor, shuffled: torc
         out = torch.empty(M, I, dtype=h.dtype, device=h.device)
         _call("tl_gemm_skinny_swiglu", _ptr(h), _ptr(shuffled), _ptr(out), M, I, K, lda, I, _stream())
         return out
+    if _rows64_ok(h, shuffled, M, K, lda) and library().tl_gemm_rows64_shares(M, 2 * I, K) > 1:
+        out = torch.empty(M, I, dtype=h.dtype, device=h.device)
+        return _rows64(h, shuffled, None, out, M, 2 * I, K, lda, I, swiglu=True)
     return silu_mul(linear(h, gate_up_weight, shuffled=shuffled))
 
 

@@ -78,10 +78,10 @@ def test_linear(dtype, M, N, Kd):
 
 
 @pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 48, 64])
-@pytest.mark.parametrize("N,Kd", [(1000, 1184), (4608, 3584), (136, 8), (50, 264)])
-def test_linear_few_rows_bfloat16(M, N, Kd, monkeypatch):
-    """The streaming MFMA kernel: every M up to 64, N no multiple of 16, K with a partial chunk."""
-    monkeypatch.setattr(K(), "SKINNY_MAX_ROWS", 64)      # also the row counts the engine gives to the library today
+@pytest.mark.parametrize("N,Kd", [(1000, 1184), (4608, 3584), (136, 8), (50, 264), (3584, 18944)])
+def test_linear_few_rows_bfloat16(M, N, Kd):
+    """The streaming MFMA kernels (up to 16 rows, and 17 to 64): N no multiple of 16 or 128, K with a
+    partial chunk, K cut into shares."""
     torch.manual_seed(M + N)
     a = torch.randn(M, Kd, device=DEV).to(torch.bfloat16)
     w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(torch.bfloat16)
@@ -89,20 +89,20 @@ def test_linear_few_rows_bfloat16(M, N, Kd, monkeypatch):
     want = a.double() @ w.double().T + b.double()
     ws = K().shuffle_weight(w)
     got = K().linear(a, w, b, out_dtype=torch.float32, shuffled=ws)
-    torch.testing.assert_close(got.double(), want, atol=2e-4, rtol=2e-4)
+    torch.testing.assert_close(got.double(), want, atol=2e-4 * math.sqrt(Kd / 1000 + 1), rtol=2e-4)
     got16 = K().linear(a, w, b, shuffled=ws)
     torch.testing.assert_close(got16.double(), want, atol=3e-2, rtol=3e-2)
     # the value of a row does not depend on the rows beside it
     alone = K().linear(a[M - 1:M].contiguous(), w, b, out_dtype=torch.float32, shuffled=ws)
     same_class = M <= 16          # up to 16 rows run the same code with the same split of K: same bits
-    torch.testing.assert_close(alone[0], got[M - 1], atol=0 if same_class else 2e-4, rtol=0 if same_class else 2e-4)
+    t = 0 if same_class else 2e-4 * math.sqrt(Kd / 1000 + 1)
+    torch.testing.assert_close(alone[0], got[M - 1], atol=t, rtol=t)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M", [1, 8, 40, 64, 200])
 @pytest.mark.parametrize("I,Kd", [(176, 64), (1184, 3584), (100, 48), (48, 136)])
-def test_swiglu_gate_up(dtype, M, I, Kd, monkeypatch):
-    monkeypatch.setattr(K(), "SKINNY_MAX_ROWS", 64)
+def test_swiglu_gate_up(dtype, M, I, Kd):
     torch.manual_seed(M + I)
     h = torch.randn(M, Kd, device=DEV).to(dtype)
     w = (torch.randn(2 * I, Kd, device=DEV) / math.sqrt(Kd) * 2).to(dtype)
