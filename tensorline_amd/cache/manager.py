@@ -23,6 +23,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Sequence
 
+import numpy as np
 import torch
 
 from tensorline_amd.cache.allocator import BlockAllocator, block_hash
@@ -50,6 +51,7 @@ class _Request:
     trimmed: list[int]                       # per group: logical pages below this are given back
     state_slot: int
     hashes: list[int] = field(default_factory=list)   # content hashes of its full, computed pages
+    arrays: list = field(default_factory=list)        # per group: the table as an int32 array, or None when stale
 
 
 class CacheManager:
@@ -175,7 +177,8 @@ class CacheManager:
         slot = self._free_slots.pop()
         for t in self.state.values():
             t[slot].zero_()
-        self._requests[rid] = _Request([[] for _ in self.groups], [0] * len(self.groups), slot)
+        self._requests[rid] = _Request([[] for _ in self.groups], [0] * len(self.groups), slot,
+                                       arrays=[None] * len(self.groups))
         return slot
 
     def state_slot(self, rid) -> int:
@@ -183,6 +186,15 @@ class CacheManager:
 
     def table(self, rid, group: int = 0) -> list[int]:
         return self._requests[rid].tables[group]
+
+    def table_array(self, rid, group: int = 0) -> np.ndarray:
+        """The table as an int32 array, rebuilt only after it changed (a step of a large batch would
+        otherwise convert every list again)."""
+        req = self._requests[rid]
+        arr = req.arrays[group]
+        if arr is None:
+            arr = req.arrays[group] = np.asarray(req.tables[group], dtype=np.int32)
+        return arr
 
     def grow(self, rid, upto: int) -> bool:
         """Make every group's table cover positions < ``upto``.  All groups or none
@@ -192,11 +204,12 @@ class CacheManager:
         needs = [max(0, want - len(t)) for t in req.tables]
         if any(n > g.allocator.num_free for n, g in zip(needs, self.groups)):
             return False
-        for n, g, t in zip(needs, self.groups, req.tables):
+        for gi, (n, g, t) in enumerate(zip(needs, self.groups, req.tables)):
             if n:
                 got = g.allocator.allocate(n)
                 assert got is not None
                 t.extend(got)
+                req.arrays[gi] = None
         return True
 
     def trim(self, rid, computed: int) -> int:
@@ -220,6 +233,7 @@ class CacheManager:
             if back:
                 g.allocator.free(back)
                 given += len(back)
+                req.arrays[gi] = None
             req.trimmed[gi] = max(req.trimmed[gi], upto_page)
         return given
 
@@ -257,6 +271,7 @@ class CacheManager:
         if table and len(table) * bs == len(tokens):
             alloc.free([table.pop()])
             req.hashes.pop()
+        req.arrays[0] = None
         return len(table) * bs
 
     def publish(self, rid, tokens: Sequence[int], computed: int) -> None:

@@ -82,13 +82,16 @@ class PackedBatch:
 
 def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[int]]], state_slots: Sequence[int],
                page_size: int, num_groups: int, scratch_page: int, vocab_size: int,
-               pad_seqs: int = 0, pad_nb: Sequence[int] | None = None, scratch_slot: int = 0) -> PackedBatch:
+               pad_seqs: int = 0, pad_nb: Sequence[int] | None = None, scratch_slot: int = 0,
+               windowed: Sequence[bool] | None = None) -> PackedBatch:
     """Flatten a step.  ``tables[s][g]`` is the page table of sequence ``s`` in group ``g`` and must
     cover positions < start + len.  With ``pad_seqs``/``pad_nb`` the batch is padded to a fixed
     shape with one-token rows that touch only the scratch page and the scratch slot."""
     S = len(entries)
     if S == 0:
         raise ValueError("a step needs at least one entry")
+    if windowed is None:
+        windowed = [True] * num_groups               # assume tables may hold pages already given back
     q_lens = [len(e.tokens) for e in entries]
     if min(q_lens) <= 0:
         raise ValueError("every entry of a step brings at least one token")
@@ -117,30 +120,48 @@ def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[
     r0 = 0
     for s, e in enumerate(entries):
         n = q_lens[s]
-        toks = np.asarray(e.tokens, dtype=np.int64)
-        if toks.min() < 0 or toks.max() >= vocab_size:
-            raise ValueError(f"request {e.rid!r}: token id outside [0, {vocab_size})")
         if e.start < 0:
             raise ValueError(f"request {e.rid!r}: negative start")
-        ids[r0:r0 + n] = toks
-        p = np.arange(e.start, e.start + n, dtype=np.int32)
-        pos[r0:r0 + n] = p
+        need_pages = -(-(e.start + n) // page_size)
+        if n == 1:                                   # a decoded token: scalars instead of arrays
+            tok = int(e.tokens[0])
+            if not 0 <= tok < vocab_size:
+                raise ValueError(f"request {e.rid!r}: token id outside [0, {vocab_size})")
+            ids[r0] = tok
+            pos[r0] = e.start
+            p = None
+        else:
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            if toks.min() < 0 or toks.max() >= vocab_size:
+                raise ValueError(f"request {e.rid!r}: token id outside [0, {vocab_size})")
+            ids[r0:r0 + n] = toks
+            p = np.arange(e.start, e.start + n, dtype=np.int32)
+            pos[r0:r0 + n] = p
         seq_of[r0:r0 + n] = s
         q_start[s] = r0
         ctx_start[s] = e.start
         slots_state[s] = state_slots[s]
-        need_pages = -(-(e.start + n) // page_size)
         for g in range(num_groups):
-            tab = np.asarray(tables[s][g], dtype=np.int32)
+            tab = tables[s][g]
+            if not isinstance(tab, np.ndarray):
+                tab = np.asarray(tab, dtype=np.int32)
             if len(tab) < need_pages:
                 raise ValueError(f"request {e.rid!r}: page table covers {len(tab) * page_size} tokens, "
                                  f"{e.start + n} are needed")
-            pages = tab[p // page_size]
-            if pages.min() < 0:
-                raise ValueError(f"request {e.rid!r}: a token of this step lies on a page already given back")
-            g_slots[g][r0:r0 + n] = pages * page_size + p % page_size
-            row = np.where(tab >= 0, tab, scratch_page)
-            g_tables[g][s, :len(row)] = row
+            if p is None:
+                page = int(tab[e.start // page_size])
+                if page < 0:
+                    raise ValueError(f"request {e.rid!r}: a token of this step lies on a page already given back")
+                g_slots[g][r0] = page * page_size + e.start % page_size
+            else:
+                pages = tab[p // page_size]
+                if pages.min() < 0:
+                    raise ValueError(f"request {e.rid!r}: a token of this step lies on a page already given back")
+                g_slots[g][r0:r0 + n] = pages * page_size + p % page_size
+            row = g_tables[g][s]
+            row[:len(tab)] = tab
+            if windowed[g]:                          # pages a window has passed: any valid page will do
+                np.putmask(row[:len(tab)], tab < 0, scratch_page)
         for w in e.want:
             if not 0 <= w < n:
                 raise ValueError(f"request {e.rid!r}: wanted place {w} is outside its {n} tokens")

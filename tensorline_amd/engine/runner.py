@@ -44,10 +44,11 @@ class ModelRunner:
     def pack(self, entries: Sequence[StepEntry], pad_seqs: int = 0, pad_nb: Sequence[int] | None = None) -> PackedBatch:
         cache = self.cache
         ngroups = len(cache.groups)
-        tables = [[cache.table(e.rid, g) for g in range(ngroups)] for e in entries]
+        tables = [[cache.table_array(e.rid, g) for g in range(ngroups)] for e in entries]
         slots = [cache.state_slot(e.rid) for e in entries]
         return pack_batch(entries, tables, slots, cache.page_size, ngroups, cache.scratch_page,
-                          self.model.vocab_size, pad_seqs=pad_seqs, pad_nb=pad_nb, scratch_slot=cache.scratch_slot)
+                          self.model.vocab_size, pad_seqs=pad_seqs, pad_nb=pad_nb, scratch_slot=cache.scratch_slot,
+                          windowed=[g.window > 0 for g in cache.groups])
 
     def context(self, packed: PackedBatch, dev: torch.Tensor) -> tuple[StepContext, list[LayerCache]]:
         def view(name: str) -> torch.Tensor:
