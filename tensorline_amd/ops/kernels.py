@@ -236,6 +236,21 @@ def _library_linear(a, weight, bias, out_dtype) -> torch.Tensor:
     """hipBLASLt through torch for many-row bfloat16 products (float32 accumulation inside)."""
     global _MM_OUT_DTYPE_OK
     wt = weight.t()
+    M, K = a.shape
+    N = weight.shape[0]
+    tiles = -(-M // 256) * -(-N // 256)
+    if out_dtype == torch.float32 and _MM_OUT_DTYPE_OK and K >= 8192 and tiles < 200:
+        # A long K with few output tiles leaves most of the 256 CUs idle in the library's product:
+        # K is cut into 2, 4 or 8 shares run as one batched product, and the shares are added in order.
+        ks = next((c for c in (2, 4, 8) if tiles * c >= 200), 8)
+        if K % (8 * ks) == 0 and a.is_contiguous():
+            kk = K // ks
+            parts = torch.bmm(a.view(M, ks, kk).transpose(0, 1), weight.view(N, ks, kk).permute(1, 2, 0),
+                              out_dtype=torch.float32)
+            y = parts.sum(0)
+            if bias is not None:
+                y.add_(bias)
+            return y
     if out_dtype == torch.float32:
         if _MM_OUT_DTYPE_OK is None:
             try:
