@@ -265,8 +265,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
 // block of 32 keys is brought into LDS once, with contiguous loads (a key row of K, a run of keys
 // of one dim of V^T), and every wave takes its MFMA fragments from there: the keys and values a
 // prompt needs are read from the cache once per 128 columns instead of once per wave, and no load
-// touches 16 separate rows.  Blocks are double-buffered: the next one is in flight while this one
-// is multiplied.  No key split: a step with prompt portions has columns enough.
+// touches 16 separate rows.  Blocks go through a ring of three LDS buffers, two blocks ahead.  No key split: a step with prompt portions has columns enough.
 template <int DC>
 __global__ __launch_bounds__(256) void attn_mfma_shared_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
@@ -280,8 +279,8 @@ __global__ __launch_bounds__(256) void attn_mfma_shared_kernel(
     constexpr int VP = 4 + 1;                 // uint4 per dim row in LDS: 32 keys + padding
     constexpr int KU = 32 * (D / 8);          // uint4 of a K block
     constexpr int VU = D * 4;                 // uint4 of a V^T block
-    __shared__ uint4 ks[2][32 * KP];
-    __shared__ uint4 vs[2][D * VP];
+    __shared__ uint4 ks[3][32 * KP];
+    __shared__ uint4 vs[3][D * VP];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int s = blockIdx.x, kvh = blockIdx.y;
@@ -383,13 +382,19 @@ __global__ __launch_bounds__(256) void attn_mfma_shared_kernel(
         }
     };
 
+    // Three LDS buffers: blocks b and b + 1 are in LDS while block b + 2 is on its way in registers,
+    // so a block's loads have a whole iteration to arrive before they are needed.
     fetch(b_lo);
     stash(0);
+    if (b_lo + 1 <= b_hi) {
+        fetch(b_lo + 1);
+        stash(1);
+    }
+    if (b_lo + 2 <= b_hi) fetch(b_lo + 2);
     __syncthreads();
     const int krow0 = 8 * (c >> 2) + (c & 3);                // key of row c in tile 0; tile 1: + 4
     int cur = 0;
     for (int b = b_lo; b <= b_hi; ++b) {
-        if (b < b_hi) fetch(b + 1);
         if (b >= wb_lo && b <= wb_hi) {
             const int kb = b << 5;
             uint4 kf0[DC], kf1[DC], vf[DB];
@@ -402,9 +407,11 @@ __global__ __launch_bounds__(256) void attn_mfma_shared_kernel(
             for (int db = 0; db < DB; ++db) vf[db] = vs[cur][(db * 16 + c) * VP + g];
             am_block<DC, NT>(kf0, kf1, vf, qf, p_col, lo_col, kb, g, scale2, m_run, l_run, acc);
         }
-        if (b < b_hi) stash(cur ^ 1);
+        const int nxt2 = (cur + 2 >= 3) ? cur - 1 : cur + 2;
+        if (b + 2 <= b_hi) stash(nxt2);                      // block b + 2: requested an iteration ago
+        if (b + 3 <= b_hi) fetch(b + 3);
         __syncthreads();
-        cur ^= 1;
+        cur = (cur + 1 >= 3) ? 0 : cur + 1;
     }
 
 #pragma unroll

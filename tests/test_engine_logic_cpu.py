@@ -2,7 +2,6 @@
 stand-ins: every way of cutting must give the plain implementation's logits."""
 import numpy as np
 import pytest
-import torch
 
 from tensorline_amd.engine.loading import load_model
 from tensorline_amd.engine.replay import TraceSession

@@ -7,7 +7,6 @@ import sys
 
 import numpy as np
 import pytest
-import torch
 
 from tests import helpers, plain
 
