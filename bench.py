@@ -25,15 +25,20 @@ if ROOT not in sys.path:
 HBM_GBPS = 8000.0
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-# layer sizes of the Qwen2.5-7B shape
+# layer sizes of the Qwen2.5 shapes; the default run is the 7B one
 SHAPE_7B = dict(vocab_size=152064, hidden_size=3584, intermediate_size=18944, num_hidden_layers=28,
                 num_attention_heads=28, num_key_value_heads=4, head_dim=128, rope_theta=1000000.0,
                 rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768)
+SHAPE_14B = dict(SHAPE_7B, hidden_size=5120, intermediate_size=13824, num_hidden_layers=48, num_attention_heads=40,
+                 num_key_value_heads=8, rms_norm_eps=1e-5)
+SHAPE_32B = dict(SHAPE_7B, hidden_size=5120, intermediate_size=27648, num_hidden_layers=64, num_attention_heads=40,
+                 num_key_value_heads=8)
+SHAPES = {"7b": SHAPE_7B, "14b": SHAPE_14B, "32b": SHAPE_32B}
 
 
-def make_config(layers: int | None):
+def make_config(layers: int | None, shape: str = "7b"):
     from tensorline_amd.config import Qwen2Config
-    d = dict(SHAPE_7B, architectures=["Qwen2ForCausalLM"])
+    d = dict(SHAPES[shape], architectures=["Qwen2ForCausalLM"])
     if layers:
         d["num_hidden_layers"] = layers
     return Qwen2Config.from_dict(d)
@@ -141,6 +146,52 @@ def bench_prefill(llm, tokens: int, reps: int, seed: int) -> dict:
     return {"s": best, "tok_s": tokens / best}
 
 
+def bench_workload(args) -> int:
+    """A serving-style run: many concurrent requests through the scheduler (continuous batching,
+    chunked prefill), as in the 14B and 32B workloads: ``--requests`` prompts of uniform random
+    length in [--prompt-min, --prompt-max], ``--output-tokens`` each, greedy or seeded temperature
+    sampling.  Prints one JSON line: generated tokens per second over the whole run."""
+    import numpy as np
+    import torch
+
+    from tensorline_amd import LLM, SamplingParams
+    cfg = make_config(args.layers, args.shape)
+    rng = np.random.default_rng(args.seed)
+    lengths = rng.integers(args.prompt_min, args.prompt_max + 1, size=args.requests)
+    prompts = [rng.integers(0, cfg.vocab_size, size=int(n)).tolist() for n in lengths]
+    max_len = args.prompt_max + args.output_tokens + 16
+    page = 16
+    llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
+              num_blocks=args.num_blocks or None, kv_mem_fraction=0.8, max_num_seqs=args.requests,
+              max_batched_tokens=2048, max_model_len=max_len, graphs=not args.no_graphs, prefix_caching=False)
+    params = [SamplingParams(max_tokens=args.output_tokens, temperature=args.temperature, top_p=1.0,
+                             stop_token_ids={-1}, seed=args.seed + i) for i in range(args.requests)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    outs = llm.generate(prompts, params)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    c = llm.counters()
+    gen = sum(len(o.token_ids) for o in outs)
+    assert all(len(o.token_ids) == args.output_tokens for o in outs) and llm.cache.all_free()
+    ttft = sorted(o.stats.ttft_s for o in outs)
+    print(json.dumps({
+        "metric": f"generated tok/s, {args.requests} concurrent requests (Qwen2.5-{args.shape.upper()} shape)",
+        "value": round(gen / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": c["steps"], "warmup": 0,
+        "ms_per_step": round(dt / max(c["steps"], 1) * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if args.dtype in ("bfloat16", "bf16") else "fp32",
+        "data": "synthetic: random weights from a seed, token ids uniform over the vocabulary",
+        "config": {"model": f"Qwen2.5-{args.shape.upper()} shape", "global_batch": args.requests, "seq_len": max_len,
+                   "parallelism": "single GPU", "layers": cfg.num_hidden_layers,
+                   "layers_of_shape": SHAPES[args.shape]["num_hidden_layers"], "prompt_min": args.prompt_min,
+                   "prompt_max": args.prompt_max, "output_tokens": args.output_tokens, "prompt_tokens": int(lengths.sum()),
+                   "temperature": args.temperature, "chunk": 2048, "kv_pages": llm.cache.num_blocks, "page_size": page,
+                   "preemptions": c["preemptions"], "graph_replays": c["graph_replays"],
+                   "ttft_p50_s": round(ttft[len(ttft) // 2], 3), "ttft_max_s": round(ttft[-1], 3),
+                   "total_s": round(dt, 2)}}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -154,16 +205,26 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (default: the 7B shape)")
+    ap.add_argument("--workload", action="store_true", help="serving-style run instead of the step benchmark")
+    ap.add_argument("--requests", type=int, default=32)
+    ap.add_argument("--prompt-min", type=int, default=256)
+    ap.add_argument("--prompt-max", type=int, default=4096)
+    ap.add_argument("--output-tokens", type=int, default=512)
+    ap.add_argument("--temperature", type=float, default=0.7)
+    ap.add_argument("--num-blocks", type=int, default=0, help="KV pages for --workload (0: 80%% of free memory)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.workload:
+        return bench_workload(args)
 
     import torch
 
     from tensorline_amd import LLM
-    cfg = make_config(args.layers)
-    full_layers = SHAPE_7B["num_hidden_layers"]
+    cfg = make_config(args.layers, args.shape)
+    full_layers = SHAPES[args.shape]["num_hidden_layers"]
     max_batch = max(args.batch, 1 if args.no_points else 64)
     max_len = args.context + 16
     page = 16
@@ -185,7 +246,7 @@ def main() -> int:
     achieved = decode_bytes(cfg, args.batch, int(main_run["mean_context"]), elem) / step_s / 1e9
     flops = prefill_flops(cfg, args.prefill_tokens)
     line = {
-        "metric": "decode tok/s @ batch 8, context 4096 (Qwen2.5-7B shape)",
+        "metric": f"decode tok/s @ batch {args.batch}, context {args.context} (Qwen2.5-{args.shape.upper()} shape)",
         "value": round(main_run["tok_s"], 1),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -198,7 +259,7 @@ def main() -> int:
         "dtype": "bf16" if elem == 2 else "fp32",
         "data": "synthetic: random weights from a seed, token ids uniform over the vocabulary",
         "config": {
-            "model": "Qwen2.5-7B shape", "global_batch": args.batch, "seq_len": args.context,
+            "model": f"Qwen2.5-{args.shape.upper()} shape", "global_batch": args.batch, "seq_len": args.context,
             "parallelism": "single GPU", "layers": cfg.num_hidden_layers, "layers_of_shape": full_layers,
             "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
             "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,

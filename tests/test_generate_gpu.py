@@ -57,6 +57,26 @@ def test_bfloat16_generation_same_with_and_without_graphs(folder_b, greedy_want)
     assert same >= 0.6 * sum(len(x) for x in want)
 
 
+def test_seeded_sampling_survives_preemption_and_batching(folder_b, greedy_want):
+    """A request's sampled tokens depend on its seed and its logits only: the same in a roomy pool, in a
+    pool so small that requests are preempted and recomputed, and alone (32-bit, so that rounding between
+    different cuttings stays far below the probabilities' spacing)."""
+    from tensorline_amd import LLM, SamplingParams
+    d, w, cfg = folder_b
+    prompts, _ = greedy_want
+    params = [SamplingParams(max_tokens=24, temperature=0.8, top_p=0.9, stop_token_ids=NO_STOP, seed=50 + i)
+              for i in range(len(prompts))]
+    roomy = LLM(d, dtype="float32", device=DEV, num_blocks=128, block_size=8)
+    a = [o.token_ids for o in roomy.generate(prompts, params)]
+    tight = LLM(d, dtype="float32", device=DEV, num_blocks=40, block_size=8, prefix_caching=False, graphs=False)
+    b = [o.token_ids for o in tight.generate(prompts, params)]
+    assert tight.counters()["preemptions"] > 0 and tight.cache.all_free()
+    assert a == b
+    alone = [roomy.generate([p], sp)[0].token_ids for p, sp in zip(prompts[:2], params[:2])]
+    assert alone == a[:2]
+    assert len({tuple(x) for x in a}) == len(a)
+
+
 def test_stream_and_abort(folder_b, greedy_want):
     from tensorline_amd import LLM, GenStats, SamplingParams
     d, w, cfg = folder_b
