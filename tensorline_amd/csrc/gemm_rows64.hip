@@ -3,39 +3,74 @@
 // (gemm_skinny.hip); what differs is how the work is cut, because with up to 64 rows the rows of A
 // weigh as much as a 128-column slab of W and must not be re-read per 16 columns.
 //
-// A work-group of eight waves owns 128 output columns (one 16-column tile per wave) and one share
-// of K.  Per step of 128 k the group brings A[0:64, k:k+128] into LDS once, with row-contiguous
-// loads by all 512 threads, and every wave multiplies it with its own W fragments, which it loads
-// straight into registers one step ahead.  LDS is double-buffered: one barrier per step.
+// A work-group of `waves` waves owns one 16-column tile per wave and one share of K.  Per step of
+// 128 k the group brings A[0:64, k:k+128] into LDS once, with row-contiguous loads by all its
+// threads, and every wave multiplies it with its own W fragments, which it loads straight into
+// registers.  Loads of A and W run several steps ahead in a ring of registers; LDS is
+// double-buffered: one barrier per step.
 //
-// K is split over the grid so that small matrices still fill 256 CUs.  With one share the result
-// is written at once; otherwise every share writes a float partial [share, M, N] and a second
-// kernel adds the shares in ascending order (and applies bias, or SiLU(gate) * up for a fused
-// gate/up matrix), so the result does not depend on timing.
+// How the work is cut decides the speed.  A CU streams weights at a bounded rate however many
+// loads its waves have in flight, so the product is as fast as the busiest CU: the cut (waves per
+// group, shares of K) is chosen so that the groups fill the 256 CUs in whole rounds with as little
+// left over as possible (r64_plan).  With one share the result is written at once; otherwise every
+// share writes a float partial [share, M, N] and a second kernel adds the shares in ascending
+// order (and applies bias, or SiLU(gate) * up for a fused gate/up matrix), so the result does not
+// depend on timing.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-#define R64_WAVES 8
 #define R64_SC 128
 #define R64_UNITS (R64_SC / 8)
 #define R64_ROWPAD 17
 #define R64_MT 4
+#ifndef R64_DEPTH
+#define R64_DEPTH 2
+#endif
+#ifndef R64_A_WEIGHT
+#define R64_A_WEIGHT 1
+#endif
+#define R64_PIECES (64 * R64_UNITS)          // 16-byte pieces of A per step
+#define R64_MIN_WAVES 4
+#define R64_MAX_WAVES 16
+#define R64_CUS 256
 
 __device__ __forceinline__ bf16x8 r64_frag(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-template <typename TO>
-__global__ __launch_bounds__(R64_WAVES * 64) void gemm_rows64_kernel(
+// Loads of one step: this thread's P pieces of A and this lane's four W fragments.  Steps are
+// clamped by the caller, so every address is valid; nothing here depends on the loaded data, so
+// the loads stay in flight until the step that uses them.
+template <int P>
+__device__ __forceinline__ void r64_issue(const bf16_t* const (&xp)[P], const uint4* w1, int step, int xunit, int K,
+                                          int last_c, uint4 (&xo)[P], uint4 (&wo)[4]) {
+    const int kbase = (step * R64_SC + xunit * 8 < K) ? step * R64_SC : 0;
+#pragma unroll
+    for (int i = 0; i < P; ++i) xo[i] = *reinterpret_cast<const uint4*>(xp[i] + kbase);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int c = step * 4 + i;
+        if (c > last_c) c = last_c;
+        wo[i] = w1[(size_t)c * 64];
+    }
+}
+
+// P: pieces of A a thread loads per step; the group has at least 1024 / P threads (a multiple of
+// 16, so that a thread's pieces all lie in one 16-byte column of the step).  Wave w of group x owns
+// tile w * gridDim.x + x: groups differ by at most one live wave.
+template <typename TO, int P, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemm_rows64_kernel(
     const bf16_t* __restrict__ A, const uint4* __restrict__ Ws, const float* __restrict__ bias, TO* __restrict__ C,
     float* __restrict__ partial, int M, int N, int K, int K32, int lda, int ldc, int steps_per_share, int ntiles) {
+    constexpr int DEPTH = R64_DEPTH;
     __shared__ uint4 xs[2][R64_MT * R64_UNITS * R64_ROWPAD];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nthreads = blockDim.x;
     const int r = lane & 15, g = lane >> 4;
     const int nsc = (K32 + 3) / 4;
     const int s0 = blockIdx.y * steps_per_share;
     const int s1 = (s0 + steps_per_share < nsc) ? s0 + steps_per_share : nsc;
-    int tile = blockIdx.x * R64_WAVES + wave;
+    int tile = wave * gridDim.x + blockIdx.x;
     const bool tile_live = tile < ntiles;
     if (!tile_live) tile = ntiles - 1;                       // loads stay in bounds; nothing is written
     const uint4* w1 = Ws + (size_t)tile * K32 * 64 + lane;
@@ -46,62 +81,60 @@ __global__ __launch_bounds__(R64_WAVES * 64) void gemm_rows64_kernel(
 #pragma unroll
     for (int i = 0; i < R64_MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // loader of A: 64 rows x 16 units = 1024 16-byte pieces, two per thread
-    const bf16_t* xp[2];
-    int xslot[2];
+    // loader of A: 64 rows x 16 units = 1024 16-byte pieces, up to P per thread
+    const bf16_t* xp[P];
+    int xslot[P];
+    bool xmine[P];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int idx = tid + 512 * i;
-        const int row = idx >> 4, unit = idx & 15;
+    for (int i = 0; i < P; ++i) {
+        const int idx = tid + nthreads * i;
+        xmine[i] = idx < R64_PIECES;
+        const int row = xmine[i] ? idx >> 4 : 0, unit = idx & 15;
         xp[i] = A + (size_t)(row < M ? row : 0) * lda + unit * 8;
         xslot[i] = ((row >> 4) * R64_UNITS + unit) * R64_ROWPAD + (row & 15);
     }
     const int xunit = tid & 15;
-    uint4 xr[2], wf[4], wn[4];
-    {
-        const int kx = s0 * R64_SC + xunit * 8;
-        const int kbase = (kx < K) ? s0 * R64_SC : 0;
+    const int nst = s1 - s0;
+    uint4 xa[DEPTH][P], wr[DEPTH][4];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) xr[i] = *reinterpret_cast<const uint4*>(xp[i] + kbase);
-        if (kx >= K) xr[0] = xr[1] = zero;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int c = s0 * 4 + i;
-            if (c > last_c) c = last_c;
-            wf[i] = w1[(size_t)c * 64];
-        }
+    for (int j = 0; j < DEPTH; ++j) {
+        const int st = (j < nst) ? s0 + j : s1 - 1;
+        r64_issue<P>(xp, w1, st, xunit, K, last_c, xa[j], wr[j]);
+        __builtin_amdgcn_sched_barrier(0);                   // oldest slot first, as in the loop below
     }
     int cur = 0;
-    for (int sc = s0; sc < s1; ++sc) {
-        xs[cur][xslot[0]] = xr[0];
-        xs[cur][xslot[1]] = xr[1];
-        __syncthreads();
-        const int sn = (sc + 1 < s1) ? sc + 1 : sc;          // past the end: the same step again, unused
-        const int kxn = sn * R64_SC + xunit * 8;
-        const int kbn = (kxn < K) ? sn * R64_SC : 0;
+    for (int base = 0; base < nst; base += DEPTH) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) xr[i] = *reinterpret_cast<const uint4*>(xp[i] + kbn);
+        for (int j = 0; j < DEPTH; ++j) {
+            const int it = base + j;
+            const int sc = (it < nst) ? s0 + it : s1 - 1;
+            // No branch in here: a step past the share's end (the step count need not be a multiple
+            // of DEPTH) runs on zeros.  Pieces of A past K count as zero too.
+            const bool xlive = it < nst && sc * R64_SC + xunit * 8 < K;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int c = sn * 4 + i;
-            if (c > last_c) c = last_c;
-            wn[i] = w1[(size_t)c * 64];
-        }
-        const int cbase = sc * 4;
-#pragma unroll
-        for (int cc = 0; cc < 4; ++cc) {
-            const bool live = cbase + cc <= last_c;          // chunks past K32 read a clamped chunk
-#pragma unroll
-            for (int mt = 0; mt < R64_MT; ++mt) {
-                uint4 xf = xs[cur][(mt * R64_UNITS + cc * 4 + g) * R64_ROWPAD + r];
-                if (!live) xf = zero;
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(r64_frag(wf[cc]), r64_frag(xf), acc[mt], 0, 0, 0);
+            for (int i = 0; i < P; ++i) {
+                uint4 x = xa[j][i];
+                if (!xlive) x = zero;
+                if (xmine[i]) xs[cur][xslot[i]] = x;
             }
-        }
-        if (kxn >= K) xr[0] = xr[1] = zero;
+            __syncthreads();
+            // chunks past K32 multiply a clamped (valid) chunk of W with pieces of A that are zero
 #pragma unroll
-        for (int i = 0; i < 4; ++i) wf[i] = wn[i];
-        cur ^= 1;
+            for (int cc = 0; cc < 4; ++cc) {
+#pragma unroll
+                for (int mt = 0; mt < R64_MT; ++mt) {
+                    const uint4 xf = xs[cur][(mt * R64_UNITS + cc * 4 + g) * R64_ROWPAD + r];
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(r64_frag(wr[j][cc]), r64_frag(xf), acc[mt], 0, 0, 0);
+                }
+            }
+            // Refill this slot of the ring only now that its values are used up, so that the slot
+            // keeps its registers over the whole loop and nothing has to wait for a copy.
+            __builtin_amdgcn_sched_barrier(0);
+            const int sn = (it + DEPTH < nst) ? s0 + it + DEPTH : s1 - 1;   // past the end: a step again, unused
+            r64_issue<P>(xp, w1, sn, xunit, K, last_c, xa[j], wr[j]);
+            __builtin_amdgcn_sched_barrier(0);
+            cur ^= 1;
+        }
     }
     if (!tile_live) return;
     // accumulator register i of lane l: C[m = mt*16 + l % 16][n = tile*16 + 4*(l / 16) + i]
@@ -142,19 +175,56 @@ __global__ void gemm_rows64_reduce_kernel(const float* __restrict__ partial, con
     C[(size_t)m * ldc + n] = tl_from_float<TO>(v);
 }
 
-// Number of shares K is cut into for a [N, K] matrix and M rows: enough work-groups to fill the
-// GPU, partial sums that stay well below the weight bytes, at least two steps per share.
-extern "C" int tl_gemm_rows64_shares(int M, int N, int K) {
-    const int groups = tl_ceil_div(tl_ceil_div(N, 16), R64_WAVES);
+// The cut of a [N, K] product with M rows: waves per group and shares of K.  The cost of a cut is
+// the work of the busiest CU in units of one wave's step (4 KB of W): whole rounds of groups over
+// the CUs, each group as slow as its waves are many, plus two steps of filling and draining per
+// group, plus (with more than one share) the second kernel and the partial sums' traffic.  The
+// group's loads of A weigh about as much as one more wave's loads of W.
+struct R64Plan {
+    int waves, shares, steps, groups_x;
+};
+
+static R64Plan r64_plan(int M, int N, int K) {
+    const int ntiles = tl_ceil_div(N, 16);
     const int nsc = tl_ceil_div(tl_ceil_div(K, 32), 4);
-    if (groups >= 256) return 1;                 // wide matrices fill the GPU without a split
-    int ks = tl_ceil_div(512, groups);
-    const int by_traffic = K / (8 * (M > 0 ? M : 1));
-    if (ks > by_traffic) ks = by_traffic;
-    if (ks > nsc / 2) ks = nsc / 2;
-    if (ks < 1) ks = 1;
-    const int steps = tl_ceil_div(nsc, ks);
-    return tl_ceil_div(nsc, steps);
+    R64Plan best{R64_MIN_WAVES, 1, nsc, tl_ceil_div(ntiles, R64_MIN_WAVES)};
+    double best_cost = 1e30;
+    const int max_shares = nsc / 2 > 1 ? nsc / 2 : 1;
+    for (int waves = R64_MIN_WAVES; waves <= R64_MAX_WAVES; ++waves) {
+        const int gx = tl_ceil_div(ntiles, waves);
+        const int live = tl_ceil_div(ntiles, gx);            // waves with a tile in the fullest group
+        for (int want = 1; want <= max_shares && want <= 64; ++want) {
+            const int steps = tl_ceil_div(nsc, want);
+            const int shares = tl_ceil_div(nsc, steps);
+            if (shares != want) continue;                     // the same cut as a smaller `want`
+            const int rounds = tl_ceil_div(gx * shares, R64_CUS);
+            double cost = (double)rounds * (live + R64_A_WEIGHT) * (steps + 2);
+            if (shares > 1) cost += 25.0 + (double)shares * (M > 0 ? M : 1) * N * 8.0 / R64_CUS / 4096.0;
+            if (cost < best_cost) {
+                best_cost = cost;
+                best = R64Plan{waves, shares, steps, gx};
+            }
+        }
+    }
+    return best;
+}
+
+// Number of shares K is cut into for a [N, K] matrix and M rows (the caller sizes the workspace by it).
+extern "C" int tl_gemm_rows64_shares(int M, int N, int K) { return r64_plan(M, N, K).shares; }
+
+template <typename TO>
+static void r64_launch(const R64Plan& p, hipStream_t stream, const bf16_t* A, const uint4* Ws, const float* bias, TO* C,
+                       float* part, int M, int N, int K, int K32, int lda, int ldc, int ntiles) {
+    dim3 grid(p.groups_x, p.shares), block(p.waves * 64);
+    if (p.waves >= 16)
+        hipLaunchKernelGGL((gemm_rows64_kernel<TO, 1, 1024>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K, K32,
+                           lda, ldc, p.steps, ntiles);
+    else if (p.waves >= 8)
+        hipLaunchKernelGGL((gemm_rows64_kernel<TO, 2, 1024>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K, K32,
+                           lda, ldc, p.steps, ntiles);
+    else
+        hipLaunchKernelGGL((gemm_rows64_kernel<TO, 4, 512>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K, K32,
+                           lda, ldc, p.steps, ntiles);
 }
 
 // A: bfloat16 [M, K], 16 < M <= 64 is what it is for (any M from 1 to 64 works); Ws: shuffled copy of
@@ -166,24 +236,20 @@ extern "C" int tl_gemm_rows64(const void* A, const void* Ws, const float* bias, 
     TL_CHECK_ARG(M >= 0 && M <= 64 && N > 0 && K > 0, "tl_gemm_rows64: bad sizes M=%d N=%d K=%d", M, N, K);
     TL_CHECK_ARG(K % 8 == 0 && lda % 8 == 0 && lda >= K, "tl_gemm_rows64: K=%d and the row stride %d must be multiples of 8", K, lda);
     TL_CHECK_ARG(((uintptr_t)A % 16) == 0 && ((uintptr_t)Ws % 16) == 0, "tl_gemm_rows64: operands must be 16-byte aligned");
-    TL_CHECK_ARG(shares == tl_gemm_rows64_shares(M, N, K), "tl_gemm_rows64: %d shares do not fit this shape", shares);
+    const R64Plan plan = r64_plan(M, N, K);
+    TL_CHECK_ARG(shares == plan.shares, "tl_gemm_rows64: %d shares do not fit this shape", shares);
     TL_CHECK_ARG(shares == 1 || partial, "tl_gemm_rows64: shares need a workspace");
     TL_CHECK_ARG(!swiglu || (N % 2 == 0 && shares > 1), "tl_gemm_rows64: the SwiGLU form needs N even and split K");
     const int n_out = swiglu ? N / 2 : N;
     TL_CHECK_ARG(ldc >= n_out && C, "tl_gemm_rows64: bad output");
+    TL_CHECK_ARG(c_dtype == TL_F32 || c_dtype == TL_BF16, "tl_gemm_rows64: unknown output dtype %d", c_dtype);
     if (M == 0) return 0;
-    const int K32 = tl_ceil_div(K, 32), nsc = tl_ceil_div(K32, 4), ntiles = tl_ceil_div(N, 16);
-    const int steps = tl_ceil_div(nsc, shares);
-    dim3 grid(tl_ceil_div(ntiles, R64_WAVES), shares), block(R64_WAVES * 64);
+    const int K32 = tl_ceil_div(K, 32), ntiles = tl_ceil_div(N, 16);
     float* part = shares > 1 ? partial : nullptr;
     if (c_dtype == TL_F32)
-        hipLaunchKernelGGL(gemm_rows64_kernel<float>, grid, block, 0, stream, (const bf16_t*)A, (const uint4*)Ws, bias,
-                           (float*)C, part, M, N, K, K32, lda, ldc, steps, ntiles);
-    else if (c_dtype == TL_BF16)
-        hipLaunchKernelGGL(gemm_rows64_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)A, (const uint4*)Ws, bias,
-                           (bf16_t*)C, part, M, N, K, K32, lda, ldc, steps, ntiles);
+        r64_launch<float>(plan, stream, (const bf16_t*)A, (const uint4*)Ws, bias, (float*)C, part, M, N, K, K32, lda, ldc, ntiles);
     else
-        return tl_fail("tl_gemm_rows64: unknown output dtype %d", c_dtype);
+        r64_launch<bf16_t>(plan, stream, (const bf16_t*)A, (const uint4*)Ws, bias, (bf16_t*)C, part, M, N, K, K32, lda, ldc, ntiles);
     TL_CHECK_LAUNCH("tl_gemm_rows64");
     if (shares > 1) {
         dim3 rgrid(tl_ceil_div(n_out, 256), M), rblock(256);
