@@ -63,6 +63,7 @@ class StepContext:
     host_q_start: list[int] = field(default_factory=list)
     host_ctx_start: list[int] = field(default_factory=list)
     host_state_slots: list[int] = field(default_factory=list)
+    logits_for_all_rows: bool = False  # logit_rows is 0, 1, .., T-1: no gather is needed
 
 
 @dataclass
@@ -78,6 +79,7 @@ class PackedBatch:
     host_q_start: list[int]
     host_ctx_start: list[int]
     host_state_slots: list[int]
+    logits_for_all_rows: bool = False
 
 
 def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[int]]], state_slots: Sequence[int],
@@ -193,4 +195,5 @@ def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[
         max_context=max(st + n for st, n in zip(starts, q_lens)), max_query_len=max(q_lens),
         decode_only=all(n == 1 for n in q_lens), num_seqs=S_pad, q_lens=q_lens, starts=starts)
     return PackedBatch(data.astype(np.int32, copy=False), T, S_pad, len(rows), offsets, group_nb, plan,
-                       [int(v) for v in q_start], [int(v) for v in ctx_start], [int(v) for v in slots_state])
+                       [int(v) for v in q_start], [int(v) for v in ctx_start], [int(v) for v in slots_state],
+                       logits_for_all_rows=rows == list(range(T)))

@@ -103,10 +103,26 @@ class DecoderModel:
         """``caches[i]`` is the view of the cache for schedule entry ``i``."""
         x = kernels.embed(ctx.ids, self.embed_table)
         pending = None
+        last = len(self.schedule) - 1
         for i, e in enumerate(self.schedule):
-            pending = self.blocks[e.layer].forward(x, pending, ctx, caches[i])
+            block = self.blocks[e.layer]
+            if getattr(block, "takes_normed_rows", None) is None:
+                pending = block.forward(x, pending, ctx, caches[i])      # a block that knows no hand-off
+                continue
+            # the norm after this block, if whoever applies it can take it as NormedRows
+            next_norm = None
+            if i < last:
+                nxt = self.blocks[self.schedule[i + 1].layer]
+                if getattr(nxt, "takes_normed_rows", lambda: False)():
+                    next_norm = nxt.mixer_norm
+            elif self.head.shuffled is not None:
+                next_norm = self.final_norm
+            pending = block.forward(x, pending, ctx, caches[i], next_norm=next_norm)
         if ctx.logit_rows.numel() == 0:
             # the residual stream is complete only after the last add; nothing reads it here
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=x.device)
-        h = self.final_norm.forward(x, pending, rows=ctx.logit_rows)
+        if isinstance(pending, kernels.NormedRows):
+            h = pending if ctx.logits_for_all_rows else pending.take(ctx.logit_rows)
+        else:
+            h = self.final_norm.forward(x, pending, rows=ctx.logit_rows)
         return self.head(h, out_dtype=torch.float32)

@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import threading
+from dataclasses import dataclass
 
 import torch
 
@@ -161,12 +162,85 @@ def _check_shuffled(shuffled: torch.Tensor, N: int, K: int) -> None:
            f"linear: the shuffled weight copy does not belong to a [{N}, {K}] matrix")
 
 
-def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None,
+@dataclass
+class NormedRows:
+    """Activations whose RMS normalisation is still owed.  ``rows`` [M, K] holds ``h * weight`` in
+    the activation dtype and ``sumsq`` [parts, M] float32 partial sums of ``h^2``, row m's in column m; the
+    product that takes them multiplies its result rows by ``1 / sqrt(sum(sumsq) / dim + eps)``,
+    which equals the product of the normalised rows because the division is one factor per row."""
+    rows: torch.Tensor
+    sumsq: torch.Tensor
+    dim: int
+    eps: float
+
+    def take(self, index: torch.Tensor) -> "NormedRows":
+        """The rows ``index`` (int tensor) only."""
+        idx = index.long()
+        return NormedRows(self.rows.index_select(0, idx), self.sumsq.index_select(1, idx), self.dim, self.eps)
+
+
+@dataclass
+class NormSink:
+    """What a product that ends a residual branch does instead of returning its result: add it to
+    ``resid`` (float32 [M, N], in place) and hand the sum on as the :class:`NormedRows` of the next
+    RMS norm (``weight`` float32 [N], ``eps``)."""
+    resid: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+
+
+class _NormArgs(ctypes.Structure):
+    _fields_ = [("ss_in", ctypes.c_void_p), ("ss_ld", ctypes.c_int), ("ss_n", ctypes.c_int),
+                ("dim", ctypes.c_float), ("eps", ctypes.c_float),
+                ("resid", ctypes.c_void_p), ("resid_ld", ctypes.c_int), ("next_weight", ctypes.c_void_p),
+                ("a_out", ctypes.c_void_p), ("a_ld", ctypes.c_int), ("ss_out", ctypes.c_void_p),
+                ("ss_out_ld", ctypes.c_int)]
+
+
+def can_defer_norm(num_rows: int, dtype: torch.dtype) -> bool:
+    """Whether the few-row products can carry the norms of a step of ``num_rows`` rows."""
+    return dtype == torch.bfloat16 and 0 < num_rows <= SKINNY_MAX_ROWS
+
+
+def _norm_args(owed: NormedRows | None, sink: NormSink | None, M: int, N: int, device):
+    """(ctypes argument, NormedRows the sink produces or None) for the few-row entry points."""
+    if owed is None and sink is None:
+        return None, None
+    na = _NormArgs()
+    produced = None
+    if owed is not None:
+        _check(owed.sumsq.dtype == torch.float32 and owed.sumsq.dim() == 2 and owed.sumsq.shape[1] == M
+               and owed.sumsq.stride(1) == 1 and owed.sumsq.stride(0) >= M,
+               "owed norm: partial sums must be float32 [parts, M]")
+        na.ss_in, na.ss_ld, na.ss_n = owed.sumsq.data_ptr(), owed.sumsq.stride(0), owed.sumsq.shape[0]
+        na.dim, na.eps = float(owed.dim), float(owed.eps)
+    if sink is not None:
+        r, w = sink.resid, sink.weight
+        _on_gpu(r, w)
+        _check(r.dtype == torch.float32 and tuple(r.shape) == (M, N) and r.stride(1) == 1,
+               f"residual sink: the residual must be float32 [{M}, {N}]")
+        _check(w.dtype == torch.float32 and w.is_contiguous() and w.numel() == N,
+               f"residual sink: the norm weight must be float32 of {N} entries")
+        parts = -(-N // 16)
+        produced = NormedRows(torch.empty(M, N, dtype=torch.bfloat16, device=device),
+                              torch.empty(parts, M, dtype=torch.float32, device=device), N, float(sink.eps))
+        na.resid, na.resid_ld, na.next_weight = r.data_ptr(), r.stride(0), w.data_ptr()
+        na.a_out, na.a_ld = produced.rows.data_ptr(), N
+        na.ss_out, na.ss_out_ld = produced.sumsq.data_ptr(), M
+    return ctypes.byref(na), produced
+
+
+def linear(a: torch.Tensor | NormedRows, weight: torch.Tensor, bias: torch.Tensor | None = None,
            out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
-           shuffled: torch.Tensor | None = None) -> torch.Tensor:
+           shuffled: torch.Tensor | None = None, sink: NormSink | None = None) -> torch.Tensor | NormedRows:
     """``a @ weight.T + bias``: a [M, K] (rows may be strided), weight [N, K], bias float32 [N].
     ``shuffled``: the copy of ``weight`` made by :func:`shuffle_weight`, which few-row bfloat16
-    products stream instead of ``weight``."""
+    products stream instead of ``weight``.  ``a`` may be :class:`NormedRows` and ``sink`` a
+    :class:`NormSink` (then the result is the next norm's :class:`NormedRows`); both need the few-row
+    kernel (:func:`can_defer_norm` rows, a shuffled copy)."""
+    owed = a if isinstance(a, NormedRows) else None
+    if owed is not None:
+        a = owed.rows
     _on_gpu(a, weight, bias, out, shuffled)
     _check(a.dim() == 2 and a.stride(1) == 1, "linear: input must be [M, K] with unit column stride")
     _check(weight.dim() == 2 and weight.is_contiguous(), "linear: weight must be a contiguous [N, K] matrix")
@@ -177,6 +251,17 @@ def linear(a: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
         _check(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == N,
                f"linear: bias must be float32 of {N} entries")
     out_dtype = out_dtype or a.dtype
+    if owed is not None or sink is not None:
+        lda = a.stride(0) if M > 1 else K
+        _check(out is None and _skinny_ok(a, shuffled, M, K, lda),
+               "linear: a deferred norm needs the few-row bfloat16 kernel (at most 16 rows, a shuffled weight copy)")
+        _check_shuffled(shuffled, N, K)
+        norm, produced = _norm_args(owed, sink, M, N, a.device)
+        if produced is None:
+            out = torch.empty(M, N, dtype=out_dtype, device=a.device)
+        _call("tl_gemm_skinny", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), F32 if out is None else _code(out, "linear output"),
+              M, N, K, lda, N, norm, _stream())
+        return produced if produced is not None else out
     if out is None:
         if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and (
                 M > ROWS64_MAX_ROWS or (M > SKINNY_MAX_ROWS and shuffled is None)):
@@ -220,7 +305,7 @@ def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled=None) -> 
     the reference uses one too: tensorline/paged.py:179-188.)"""
     if _skinny_ok(a, shuffled, M, K, lda):
         _call("tl_gemm_skinny", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), _code(out, "linear output"),
-              M, N, K, lda, ldc, _stream())
+              M, N, K, lda, ldc, None, _stream())
         return out
     if _rows64_ok(a, shuffled, M, K, lda):
         return _rows64(a, shuffled, bias, out, M, N, K, lda, ldc, swiglu=False)
@@ -268,9 +353,14 @@ def _library_linear(a, weight, bias, out_dtype) -> torch.Tensor:
     return y
 
 
-def swiglu_gate_up(h: torch.Tensor, gate_up_weight: torch.Tensor, shuffled: torch.Tensor | None = None) -> torch.Tensor:
+def swiglu_gate_up(h: torch.Tensor | NormedRows, gate_up_weight: torch.Tensor,
+                   shuffled: torch.Tensor | None = None) -> torch.Tensor:
     """``silu(h Wg^T) * (h Wu^T)`` for a fused [2I, K] weight (gate rows first): one kernel for
-    few-row bfloat16 batches (it streams the ``shuffled`` copy), product then SiLU-multiply otherwise."""
+    few-row bfloat16 batches (it streams the ``shuffled`` copy), product then SiLU-multiply otherwise.
+    ``h`` may be :class:`NormedRows` (few-row kernel only)."""
+    owed = h if isinstance(h, NormedRows) else None
+    if owed is not None:
+        h = owed.rows
     _on_gpu(h, gate_up_weight, shuffled)
     _check(h.dim() == 2 and h.stride(1) == 1 and gate_up_weight.dim() == 2 and gate_up_weight.is_contiguous()
            and gate_up_weight.shape[0] % 2 == 0 and gate_up_weight.shape[1] == h.shape[1], "swiglu_gate_up: bad shapes")
@@ -281,8 +371,12 @@ def swiglu_gate_up(h: torch.Tensor, gate_up_weight: torch.Tensor, shuffled: torc
         _check_shuffled(shuffled, 2 * I, K)
     if _skinny_ok(h, shuffled, M, K, lda) and I % 16 == 0:
         out = torch.empty(M, I, dtype=h.dtype, device=h.device)
-        _call("tl_gemm_skinny_swiglu", _ptr(h), _ptr(shuffled), _ptr(out), M, I, K, lda, I, _stream())
+        norm, _ = _norm_args(owed, None, M, 2 * I, h.device)
+        _call("tl_gemm_skinny_swiglu", _ptr(h), _ptr(shuffled), _ptr(out), M, I, K, lda, I, norm, _stream())
         return out
+    if owed is not None:
+        # the few-row kernel pairs gate and up tiles only for I a multiple of 16: scale the product's rows instead
+        return silu_mul(linear(owed, gate_up_weight, shuffled=shuffled))
     if _rows64_ok(h, shuffled, M, K, lda) and library().tl_gemm_rows64_shares(M, 2 * I, K) > 1:
         out = torch.empty(M, I, dtype=h.dtype, device=h.device)
         return _rows64(h, shuffled, None, out, M, 2 * I, K, lda, I, swiglu=True)
@@ -300,13 +394,17 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, who: str) -> 
            f"{who}: value cache must be contiguous [pages, nkv, d, page] matching the key cache")
 
 
-def qkv_rope_store(h: torch.Tensor, shuffled: torch.Tensor, bias: torch.Tensor | None, pos: torch.Tensor,
+def qkv_rope_store(h: torch.Tensor | NormedRows, shuffled: torch.Tensor, bias: torch.Tensor | None, pos: torch.Tensor,
                    inv_freq: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                    k_cache: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor) -> torch.Tensor | None:
     """The projection, position encoding and cache write of a decode step in one kernel: returns the
     rotated queries [M, nq*d]; rotated keys and the values go into the cache at ``slots``.  Returns
     None when the kernel does not take the case (then the three separate kernels run): it needs
-    bfloat16, at most 16 rows, a head size that is a multiple of 32 and full-width rotation."""
+    bfloat16, at most 16 rows, a head size that is a multiple of 32 and full-width rotation.
+    ``h`` may be :class:`NormedRows`."""
+    owed = h if isinstance(h, NormedRows) else None
+    if owed is not None:
+        h = owed.rows
     M, K = h.shape
     N = (num_heads + 2 * num_kv_heads) * head_dim
     if not (h.dtype == torch.bfloat16 and shuffled is not None and M <= 16 and head_dim % 32 == 0
@@ -322,9 +420,10 @@ def qkv_rope_store(h: torch.Tensor, shuffled: torch.Tensor, bias: torch.Tensor |
     if bias is not None:
         _check(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == N, "qkv_rope_store: bad bias")
     q = torch.empty(M, num_heads * head_dim, dtype=h.dtype, device=h.device)
+    norm, _ = _norm_args(owed, None, M, N, h.device)
     _call("tl_gemm_skinny_qkv_rope", _ptr(h), _ptr(shuffled), _ptr(bias), _ptr(pos), _ptr(inv_freq), _ptr(slots),
           _ptr(q), _ptr(k_cache), _ptr(v_cache), M, K, h.stride(0) if M > 1 else K, num_heads, num_kv_heads,
-          head_dim, k_cache.shape[1], _stream())
+          head_dim, k_cache.shape[1], norm, _stream())
     return q
 
 

@@ -69,7 +69,11 @@ class PagedAttention(Part):
         return None
 
     # ---- one step ------------------------------------------------------------------------
-    def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
+    @property
+    def defers_norm(self) -> bool:
+        return self.qkv.shuffled is not None and self.o_proj.shuffled is not None
+
+    def forward(self, h, ctx, cache, sink=None):
         nkv_local = self.num_kv_heads if self.kv_proj else 0
         write = cache.write and self.kv_proj
         qkv = None
@@ -85,4 +89,4 @@ class PagedAttention(Part):
                                     self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
                                     window=self.window, q_start=ctx.q_start, ctx_start=ctx.ctx_start,
                                     plan=ctx.attention_plan)
-        return self.o_proj(o, out_dtype=torch.float32)
+        return self.o_proj(o, out_dtype=torch.float32, sink=sink)

@@ -34,6 +34,14 @@ class Part:
         """Device tensors this part keeps (for byte accounting)."""
         return []
 
+    # Optional hand-off of the norms to the products around them (few-row bfloat16 steps).  A mixer
+    # or feed-forward that sets ``defers_norm`` takes :class:`tensorline_amd.ops.kernels.NormedRows`
+    # as its input and a ``sink`` (:class:`tensorline_amd.ops.kernels.NormSink`) keyword: with a sink
+    # its last product adds into the residual and returns the next norm's NormedRows instead of its
+    # own output.  A norm that can be handed off this way returns (weight, eps) from ``deferrable()``.
+    # Parts without these never see either object.
+    defers_norm = False
+
 
 class Linear:
     """``y = x W^T + b`` with W [out, in] as checkpoints store it (reference: tensorline/quant.py:3)."""
@@ -65,8 +73,8 @@ class Linear:
     def tensors_kept(self) -> list[torch.Tensor]:
         return [t for t in (self.weight, self.bias, self.shuffled) if t is not None]
 
-    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
-        return kernels.linear(x, self.weight, self.bias, out_dtype=out_dtype, shuffled=self.shuffled)
+    def __call__(self, x, out_dtype: torch.dtype | None = None, sink=None):
+        return kernels.linear(x, self.weight, self.bias, out_dtype=out_dtype, shuffled=self.shuffled, sink=sink)
 
 
 def fuse_linears(name: str, parts: list[Linear]) -> Linear:

@@ -37,6 +37,10 @@ class SwiGLU(Part):
     def weight_tensors(self):
         return self.gate_up.tensors_kept() + self.down.tensors_kept()
 
-    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+    @property
+    def defers_norm(self) -> bool:
+        return self.gate_up.shuffled is not None and self.down.shuffled is not None
+
+    def forward(self, h, ctx, sink=None):
         act = kernels.swiglu_gate_up(h, self.gate_up.weight, self.gate_up.shuffled)
-        return self.down(act, out_dtype=torch.float32)
+        return self.down(act, out_dtype=torch.float32, sink=sink)

@@ -31,6 +31,10 @@ class RMSNorm(Part):
     def weight_tensors(self):
         return [self.weight]
 
+    def deferrable(self) -> tuple[torch.Tensor, float]:
+        """(weight, eps): all a product needs to carry this norm (see ``Part.defers_norm``)."""
+        return self.weight, self.eps
+
     def forward(self, x: torch.Tensor, residual: torch.Tensor | None = None,
                 rows: torch.Tensor | None = None) -> torch.Tensor:
         return kernels.add_rmsnorm(x, residual, self.weight, self.eps, self.dtype, rows=rows)

@@ -174,6 +174,41 @@ def test_parts_alone(folder_b):
         cache.release("a")
 
 
+def test_decode_steps_hand_norms_to_the_products(folder_b, monkeypatch):
+    """bfloat16 steps of few rows run one norm kernel only (the first layer's first norm): the other
+    norms ride on the products around them.  The logits agree with the same step run with a norm
+    kernel for every norm, whether all rows or some are wanted."""
+    from tensorline_amd.cache.manager import CacheManager
+    from tensorline_amd.engine.batch import StepEntry
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.runner import ModelRunner
+    from tensorline_amd.ops import kernels
+    d, w, cfg = folder_b
+    model, mc = load_model(d, "bfloat16", DEV)
+    cache = CacheManager(model.cache_needs(), model.schedule, model.state_needs(), page_size=8, num_blocks=32,
+                         max_requests=4, dtype=torch.bfloat16, device=DEV)
+    runner = ModelRunner(model, cache)
+    calls = []
+    real = kernels.add_rmsnorm
+    monkeypatch.setattr(kernels, "add_rmsnorm", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    prompts = helpers.prompts_for("B", [9, 5, 2], seed=4)
+    for i, p in enumerate(prompts):
+        cache.add_request(i)
+        cache.grow(i, len(p))
+    for want_all in (True, False):
+        entries = [StepEntry(i, p, 0, list(range(len(p))) if want_all else [len(p) - 1]) for i, p in enumerate(prompts)]
+        calls.clear()
+        got = runner.step(entries)
+        assert len(calls) == 1
+        with monkeypatch.context() as m:
+            m.setattr(kernels, "can_defer_norm", lambda rows, dtype: False)
+            calls.clear()
+            ref = runner.step(entries)
+            assert len(calls) == 2 * mc.num_hidden_layers + 1
+        torch.testing.assert_close(got, ref, atol=2e-2, rtol=2e-2)
+        assert (got.argmax(-1) == ref.argmax(-1)).float().mean() > 0.8
+
+
 def test_toy_mixer_with_state_registers_and_steps(tmp_path):
     """A mixer defined here, with per-request state of fixed size, is registered, built into a model
     beside the framework's own parts and stepped, without a change to the framework's files."""

@@ -198,6 +198,90 @@ def test_fused_projection_rotation_and_cache_write(M, nq, nkv, d, Kd):
     assert K().qkv_rope_store(h, K().shuffle_weight(w), b, pos, inv_freq[: d // 4].contiguous(), nq, nkv, d, kc, vc, slots) is None
 
 
+def _normed_rows(h, gamma, eps, parts):
+    """NormedRows of float rows ``h`` as a product's residual sink would leave them, with the sum of
+    squares cut into ``parts`` uneven partials."""
+    M, H = h.shape
+    cuts = sorted(set([0, H] + torch.randint(1, H, (parts - 1,)).tolist()))
+    ss = torch.stack([(h[:, a:b].double() ** 2).sum(1) for a, b in zip(cuts[:-1], cuts[1:])], 0).float()
+    return K().NormedRows((h * gamma).to(torch.bfloat16), ss.contiguous(), H, eps)
+
+
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("N,Kd,parts", [(176, 64, 4), (1000, 1184, 74), (3584, 3584, 224), (50, 264, 1)])
+def test_products_apply_an_owed_norm(M, N, Kd, parts):
+    """A product of rows h * g with the division by rms(h) owed equals the product of RMSNorm(h) * g:
+    plain, gate/up with SiLU, and q/k/v with rotation and cache write."""
+    torch.manual_seed(M * 1000 + N)
+    eps = 1e-5
+    h = torch.randn(M, Kd, device=DEV) * torch.logspace(-1, 2, M, device=DEV)[:, None]   # rows of very different size
+    gamma = 1 + 0.1 * torch.randn(Kd, device=DEV)
+    owed = _normed_rows(h, gamma, eps, parts)
+    rstd = 1 / torch.sqrt((h.double() ** 2).mean(1, keepdim=True) + eps)
+    x = owed.rows.double() * rstd                        # what the product must multiply, given the rounded rows
+    w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(torch.bfloat16)
+    b = torch.randn(N, device=DEV)
+    sh = K().shuffle_weight(w)
+    got = K().linear(owed, w, b, out_dtype=torch.float32, shuffled=sh)
+    torch.testing.assert_close(got.double(), x @ w.double().T + b.double(), atol=2e-3, rtol=2e-3)
+    if N % 32 == 0:
+        act = K().swiglu_gate_up(owed, w, sh)
+        y = x @ w.double().T
+        want = torch.nn.functional.silu(y[:, :N // 2]) * y[:, N // 2:]
+        torch.testing.assert_close(act.double(), want, atol=2e-2, rtol=2e-2)
+    with pytest.raises(K().KernelError, match="few-row"):
+        K().linear(owed, w, b, out_dtype=torch.float32, shuffled=None)
+
+
+def test_fused_projection_applies_an_owed_norm():
+    torch.manual_seed(3)
+    M, nq, nkv, d, Kd, bs, pages, eps = 5, 6, 2, 32, 192, 8, 12, 1e-6
+    N = (nq + 2 * nkv) * d
+    h = torch.randn(M, Kd, device=DEV) * 30
+    gamma = 1 + 0.1 * torch.randn(Kd, device=DEV)
+    owed = _normed_rows(h, gamma, eps, 12)
+    x = (owed.rows.double() / torch.sqrt((h.double() ** 2).mean(1, keepdim=True) + eps)).to(torch.bfloat16)
+    w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(torch.bfloat16)
+    b = torch.randn(N, device=DEV)
+    pos = torch.randint(0, 4000, (M,), dtype=torch.int32, device=DEV)
+    slots = torch.randperm(pages * bs, device=DEV)[:M].to(torch.int32)
+    inv_freq = (1e6 ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)).float().to(DEV)
+    out = []
+    for inp in (owed, x):
+        kc = torch.zeros(pages, bs, nkv, d, device=DEV, dtype=torch.bfloat16)
+        vc = torch.zeros(pages, nkv, d, bs, device=DEV, dtype=torch.bfloat16)
+        q = K().qkv_rope_store(inp, K().shuffle_weight(w), b, pos, inv_freq, nq, nkv, d, kc, vc, slots)
+        out.append((q, kc, vc))
+    for a, c in zip(out[0], out[1]):                     # against the same kernel on rows normalised beforehand
+        torch.testing.assert_close(a.float(), c.float(), atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("M", [1, 6, 16])
+@pytest.mark.parametrize("N,Kd", [(176, 64), (1000, 1184), (3584, 18944), (40, 264)])
+def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
+    torch.manual_seed(M + N)
+    eps = 1e-6
+    a = torch.randn(M, Kd, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(torch.bfloat16)
+    b = torch.randn(N, device=DEV)
+    gamma = 1 + 0.1 * torch.randn(N, device=DEV)
+    resid0 = torch.randn(M, N, device=DEV) * 5
+    resid = resid0.clone()
+    nxt = K().linear(a, w, b, out_dtype=torch.float32, shuffled=K().shuffle_weight(w), sink=K().NormSink(resid, gamma, eps))
+    want = resid0.double() + a.double() @ w.double().T + b.double()
+    torch.testing.assert_close(resid.double(), want, atol=1e-3, rtol=1e-4)
+    assert isinstance(nxt, K().NormedRows) and nxt.dim == N and nxt.eps == eps
+    torch.testing.assert_close(nxt.rows.float(), (resid * gamma).to(torch.bfloat16).float(), atol=0, rtol=2 ** -7)
+    assert tuple(nxt.sumsq.shape) == (-(-N // 16), M)
+    torch.testing.assert_close(nxt.sumsq.double().sum(0), (resid.double() ** 2).sum(1), atol=0, rtol=1e-5)
+    # handed on: the next product's result equals that of the norm kernel followed by the product
+    w2 = (torch.randn(48, N, device=DEV) / math.sqrt(N)).to(torch.bfloat16)
+    got = K().linear(nxt, w2, None, out_dtype=torch.float32, shuffled=K().shuffle_weight(w2))
+    x = K().add_rmsnorm(resid.clone(), None, gamma, eps, torch.bfloat16)
+    want2 = K().linear(x, w2, None, out_dtype=torch.float32, shuffled=K().shuffle_weight(w2))
+    torch.testing.assert_close(got, want2, atol=2e-2, rtol=2e-2)
+
+
 def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False, path=None, split_keys=None):
     """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries."""
     torch.manual_seed(seed)
