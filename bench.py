@@ -163,7 +163,8 @@ def bench_workload(args) -> int:
     page = 16
     llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
               num_blocks=args.num_blocks or None, kv_mem_fraction=0.8, max_num_seqs=args.requests,
-              max_batched_tokens=2048, max_model_len=max_len, graphs=not args.no_graphs, prefix_caching=False)
+              max_batched_tokens=2048, max_model_len=max_len, graphs=not args.no_graphs, prefix_caching=False,
+              tune_library=not args.no_tune)
     params = [SamplingParams(max_tokens=args.output_tokens, temperature=args.temperature, top_p=1.0,
                              stop_token_ids={-1}, seed=args.seed + i) for i in range(args.requests)]
     torch.cuda.synchronize()
@@ -204,6 +205,7 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--no-tune", action="store_true", help="keep the library's heuristic choice of kernels for prompt portions")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (default: the 7B shape)")
     ap.add_argument("--workload", action="store_true", help="serving-style run instead of the step benchmark")
@@ -230,7 +232,8 @@ def main() -> int:
     page = 16
     llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
               num_blocks=max_batch * (-(-max_len // page)) + 8, max_num_seqs=max_batch, max_batched_tokens=2048,
-              max_model_len=max_len, graphs=not args.no_graphs, graph_warmup_tokens=0, prefix_caching=False)
+              max_model_len=max_len, graphs=not args.no_graphs, graph_warmup_tokens=0, prefix_caching=False,
+              tune_library=not args.no_tune)
     elem = 2 if args.dtype in ("bfloat16", "bf16") else 4
     dtype_key = "bfloat16" if elem == 2 else "float32"
 
@@ -264,7 +267,7 @@ def main() -> int:
             "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
             "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "page_size": page,
-            "prefill_tokens": args.prefill_tokens, "graphs": not args.no_graphs, "sampling": "greedy",
+            "prefill_tokens": args.prefill_tokens, "graphs": not args.no_graphs, "library_tuning": not args.no_tune, "sampling": "greedy",
             "decode_graph_replays": main_run["graph_replays"], "mean_context": round(main_run["mean_context"], 1),
         },
         "prefill": {"value": round(pre["tok_s"], 1), "tokens": args.prefill_tokens, "ms": round(pre["s"] * 1e3, 3),

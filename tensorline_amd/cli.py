@@ -31,6 +31,8 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--graph-warmup-tokens", type=int, default=512,
                     help="capture the decode graphs before serving (0 = at first use)")
     ap.add_argument("--no-prefix-caching", action="store_true", help="never reuse KV pages across requests")
+    ap.add_argument("--tune-library", action="store_true",
+                    help="at start-up, let the library pick its kernels for full prompt portions by measurement")
 
 
 def _make_llm(a):
@@ -40,7 +42,8 @@ def _make_llm(a):
     return LLM(a.model, device=a.device, dtype=a.dtype, max_num_seqs=a.max_num_seqs,
                max_batched_tokens=a.max_batched_tokens, num_blocks=a.num_blocks, kv_cache_gb=a.kv_cache_gb,
                block_size=a.block_size, max_model_len=a.max_model_len, graphs=not a.no_graphs,
-               graph_warmup_tokens=a.graph_warmup_tokens, prefix_caching=not a.no_prefix_caching)
+               graph_warmup_tokens=a.graph_warmup_tokens, prefix_caching=not a.no_prefix_caching,
+               tune_library=a.tune_library)
 
 
 def cmd_generate(a) -> int:

@@ -60,6 +60,8 @@ class LLM:
         self.cache = CacheManager(self.model.cache_needs(), self.model.schedule, self.model.state_needs(),
                                   page_size=ec.block_size, num_blocks=num_blocks, max_requests=ec.max_num_seqs,
                                   dtype=self.model.dtype, device=device, prefix_caching=ec.prefix_caching)
+        if ec.tune_library and self.model.dtype == torch.bfloat16:
+            self.model.tune_library(ec.max_batched_tokens)
         runner = None
         if ec.graphs:
             from tensorline_amd.engine.graphs import GraphRunner

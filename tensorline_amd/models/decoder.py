@@ -99,6 +99,20 @@ class DecoderModel:
         return out
 
     # ---- one step ------------------------------------------------------------------------
+    def tune_library(self, rows: int) -> int:
+        """Let the library choose its kernels by measurement for steps of ``rows`` tokens (a full
+        prompt portion): one search per distinct product shape.  Returns how many were searched."""
+        seen, done = set(), 0
+        for block in self.blocks:
+            for part in block.parts():
+                for weight, out_dtype in getattr(part, "library_products", lambda: [])():
+                    key = (tuple(weight.shape), weight.dtype, out_dtype)
+                    if key in seen:
+                        continue
+                    seen.add(key)
+                    done += bool(kernels.tune_library_linear(rows, weight, out_dtype))
+        return done
+
     def forward(self, ctx, caches) -> torch.Tensor:
         """``caches[i]`` is the view of the cache for schedule entry ``i``."""
         x = kernels.embed(ctx.ids, self.embed_table)

@@ -353,6 +353,33 @@ def _library_linear(a, weight, bias, out_dtype) -> torch.Tensor:
     return y
 
 
+def tune_library_linear(rows: int, weight: torch.Tensor, out_dtype: torch.dtype, seconds: float = 2.0) -> bool:
+    """Have the library pick its kernel for the ``[rows, K] x [N, K]^T`` product by measurement
+    (torch's TunableOp searches the hipBLASLt and rocBLAS solutions once and keeps the fastest for
+    later calls of that shape) instead of by its heuristic: at 2,048 rows and the widths of a 7B
+    model the heuristic's choice reaches about 1.0 PFLOP/s, the measured one 1.25.  Only the shape
+    given is searched, here and now; other shapes keep the heuristic and are never searched at a
+    request's cost.  Returns False when this torch has no TunableOp or the product does not go to
+    the library."""
+    tn = getattr(torch.cuda, "tunable", None)
+    if tn is None or weight.dtype != torch.bfloat16 or rows <= ROWS64_MAX_ROWS:
+        return False
+    _on_gpu(weight)
+    tn.enable(True)
+    if hasattr(tn, "write_file_on_exit"):
+        tn.write_file_on_exit(False)
+    tn.set_max_tuning_duration(int(seconds * 1000))
+    tn.set_max_tuning_iterations(50)
+    a = torch.randn(rows, weight.shape[1], device=weight.device).to(torch.bfloat16)
+    tn.tuning_enable(True)
+    try:
+        _library_linear(a, weight, None, out_dtype)
+        torch.cuda.synchronize(weight.device)
+    finally:
+        tn.tuning_enable(False)
+    return True
+
+
 def swiglu_gate_up(h: torch.Tensor | NormedRows, gate_up_weight: torch.Tensor,
                    shuffled: torch.Tensor | None = None) -> torch.Tensor:
     """``silu(h Wg^T) * (h Wu^T)`` for a fused [2I, K] weight (gate rows first): one kernel for

@@ -69,6 +69,9 @@ class PagedAttention(Part):
         return None
 
     # ---- one step ------------------------------------------------------------------------
+    def library_products(self):
+        return [(self.qkv.weight, self.dtype), (self.o_proj.weight, torch.float32)]
+
     @property
     def defers_norm(self) -> bool:
         return self.qkv.shuffled is not None and self.o_proj.shuffled is not None

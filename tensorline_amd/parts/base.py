@@ -34,6 +34,10 @@ class Part:
         """Device tensors this part keeps (for byte accounting)."""
         return []
 
+    def library_products(self) -> list[tuple[torch.Tensor, torch.dtype]]:
+        """(weight, output dtype) of the products this part hands to the library in many-row steps."""
+        return []
+
     # Optional hand-off of the norms to the products around them (few-row bfloat16 steps).  A mixer
     # or feed-forward that sets ``defers_norm`` takes :class:`tensorline_amd.ops.kernels.NormedRows`
     # as its input and a ``sink`` (:class:`tensorline_amd.ops.kernels.NormSink`) keyword: with a sink

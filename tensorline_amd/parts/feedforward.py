@@ -37,6 +37,9 @@ class SwiGLU(Part):
     def weight_tensors(self):
         return self.gate_up.tensors_kept() + self.down.tensors_kept()
 
+    def library_products(self):
+        return [(self.gate_up.weight, self.dtype), (self.down.weight, torch.float32)]
+
     @property
     def defers_norm(self) -> bool:
         return self.gate_up.shuffled is not None and self.down.shuffled is not None

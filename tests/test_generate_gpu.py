@@ -319,3 +319,20 @@ def test_command_line_generate(folder_b, greedy_want):
     recs = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")]
     assert [r["token_ids"] for r in recs] == want[1:3]
     assert all(r["finish_reason"] == "length" and r["completion_tokens"] == 24 for r in recs)
+
+
+def test_library_tuning_keeps_results(folder_b):
+    """Letting the library choose its kernels by measurement changes which kernel runs, not what a
+    prompt portion computes."""
+    from tensorline_amd import LLM, SamplingParams
+    d, w, cfg = folder_b
+    prompt = helpers.prompts_for("B", [150], seed=9)
+    sp = SamplingParams(max_tokens=6, stop_token_ids=NO_STOP)
+    plainly = LLM(d, dtype="bfloat16", device=DEV, num_blocks=64, block_size=8, max_batched_tokens=128)
+    want = plainly.generate(prompt, sp)[0].token_ids
+    tuned = LLM(d, dtype="bfloat16", device=DEV, num_blocks=64, block_size=8, max_batched_tokens=128, tune_library=True)
+    try:
+        assert tuned.model.tune_library(128) >= 1
+        assert tuned.generate(prompt, sp)[0].token_ids == want
+    finally:
+        torch.cuda.tunable.enable(False)
