@@ -260,27 +260,120 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     }
 }
 
-// A variant for steps with prompt portions: a work-group of four waves owns 128 consecutive
-// columns of one (sequence, key/value head), 32 per wave, and walks the key blocks together.  Each
-// block of 32 keys is brought into LDS once, with contiguous loads (a key row of K, a run of keys
-// of one dim of V^T), and every wave takes its MFMA fragments from there: the keys and values a
-// prompt needs are read from the cache once per 128 columns instead of once per wave, and no load
-// touches 16 separate rows.  Blocks go through a ring of three LDS buffers, two blocks ahead.  No key split: a step with prompt portions has columns enough.
+// The same block of 32 keys with the fragments taken from LDS where they are used: kt points at
+// the block's 32 key rows (KP units each) in matrix-core order (row c of score tile 0, which is key
+// 8 (c / 4) + c % 4, in LDS row c, row c of tile 1 in LDS row 16 + c: the 16 lanes of a read then
+// take 16 consecutive rows, which the one unit of padding spreads over all banks), vt at the
+// block's 4 units of dim row 0 (VP units per dim).  All score tiles first, then the softmax of each column tile, then all P*V products, so
+// that key fragments are dead before value fragments are read: few registers are live at once.
+template <int DC, int NT, int KP, int VP>
+__device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, const uint4 (*qf)[DC], const int* p_col,
+                                             const int* lo_col, int kb, int c, int g, float scale2, float* m_run,
+                                             float* l_run, f32x4 (*acc)[DC * 2]) {
+    constexpr int DB = DC * 2;
+    const int key_base = kb + 8 * g;
+    f32x4 st0[NT], st1[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) st0[j] = st1[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) {
+        const uint4 k0 = kt[c * KP + dc * 4 + g];
+        const uint4 k1 = kt[(16 + c) * KP + dc * 4 + g];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            st0[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(k0), am_frag(qf[j][dc]), st0[j], 0, 0, 0);
+            st1[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(k1), am_frag(qf[j][dc]), st1[j], 0, 0, 0);
+        }
+    }
+    uint4 pf[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        float sv[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sv[i] = st0[j][i] * scale2;
+            sv[4 + i] = st1[j][i] * scale2;
+        }
+        const bool edge = (kb + 31 > p_col[j]) || (kb < lo_col[j]);
+        if (__any(edge)) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int key = key_base + i;
+                if (key > p_col[j] || key < lo_col[j]) sv[i] = -INFINITY;
+            }
+        }
+        float bmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 16, TL_WAVE));
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, TL_WAVE));
+        const float m_new = fmaxf(m_run[j], bmax);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const bool moved = m_new > m_run[j];
+        float pr[8], psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pr[i] = __builtin_amdgcn_exp2f(sv[i] - m_safe);
+            psum += pr[i];
+        }
+        pf[j].x = am_pack2(pr[0], pr[1]);
+        pf[j].y = am_pack2(pr[2], pr[3]);
+        pf[j].z = am_pack2(pr[4], pr[5]);
+        pf[j].w = am_pack2(pr[6], pr[7]);
+        if (__any(moved)) {
+            const float alpha = __builtin_amdgcn_exp2f(m_run[j] - m_safe);
+            l_run[j] = l_run[j] * alpha + psum;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                acc[j][db][0] *= alpha;
+                acc[j][db][1] *= alpha;
+                acc[j][db][2] *= alpha;
+                acc[j][db][3] *= alpha;
+            }
+        } else {
+            l_run[j] += psum;
+        }
+        m_run[j] = m_new;
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+        const uint4 v = vt[(db * 16 + c) * VP + g];
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+            acc[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(v), am_frag(pf[j]), acc[j][db], 0, 0, 0);
+    }
+}
+
+// The kernel for steps with prompt portions.  A work-group of four waves owns 128 consecutive
+// columns of one (sequence, key/value head), 32 per wave, and walks the keys together in tiles of
+// 64.  A tile is brought into LDS once, with contiguous loads (whole key rows of K, runs of keys of
+// one dim of V^T), and every wave takes its MFMA fragments from there: keys and values are read
+// from the cache once per 128 columns, and a wave holds no copy of them in registers, so two
+// work-groups fit on a CU and one computes while the other waits.  Two LDS buffers: the loads of
+// tile t + 1 are in flight (in registers) while tile t is multiplied, and go to the other buffer
+// before the one barrier of the iteration.  The sequence's page ids are copied to LDS first, so a
+// tile's addresses depend on no load from memory.  Pages must hold a power of two of tokens (at
+// least 8; 2^bs_shift): an 8-key run of V^T then lies in one page and a page id is a shift away.
+// No key split: a step with prompt portions has columns enough.
+#define AT_KEYS 64
+// LDS row of key k of a tile (see am_block_lds)
+__device__ __forceinline__ int at_lds_row(int k) {
+    return (k & 32) + ((k & 4) << 2) + ((k & 24) >> 1) + (k & 3);
+}
+
 template <int DC>
-__global__ __launch_bounds__(256) void attn_mfma_shared_kernel(
+__global__ __launch_bounds__(256, 2) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int nq, int nkv, int bs,
-    int window, float scale) {
+    int bs_shift, int window, float scale) {
     constexpr int NT = 2;
     constexpr int D = DC * 32;
     constexpr int DB = D / 16;
     constexpr int KP = D / 8 + 1;             // uint4 per key row in LDS (one of padding)
-    constexpr int VP = 4 + 1;                 // uint4 per dim row in LDS: 32 keys + padding
-    constexpr int KU = 32 * (D / 8);          // uint4 of a K block
-    constexpr int VU = D * 4;                 // uint4 of a V^T block
-    __shared__ uint4 ks[3][32 * KP];
-    __shared__ uint4 vs[3][D * VP];
+    constexpr int VP = AT_KEYS / 8 + 1;       // uint4 per dim row in LDS: 64 keys + padding
+    extern __shared__ uint4 at_smem[];
+    uint4* ks = at_smem;                                   // [2][AT_KEYS * KP]
+    uint4* vs = at_smem + 2 * AT_KEYS * KP;                // [2][D * VP]
+    int* tab = reinterpret_cast<int*>(vs + 2 * D * VP);    // page ids of the sequence, as far as needed
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int s = blockIdx.x, kvh = blockIdx.y;
@@ -290,11 +383,37 @@ __global__ __launch_bounds__(256) void attn_mfma_shared_kernel(
     const int n = q_start[s + 1] - r0;
     const int start = ctx_start[s];
     const int ncols = n * G;
-    const int wg_col0 = blockIdx.z * 128;
+    // the groups with the most keys (the last columns) start first
+    const int wg_col0 = (int)(gridDim.z - 1 - blockIdx.z) * 128;
     if (wg_col0 >= ncols) return;             // the whole work-group leaves: no barrier is missed
-    const int32_t* table = tables + (size_t)s * NB;
     const int col0 = wg_col0 + wave * 32;
     const bool wave_active = col0 < ncols;
+
+    // key range of the work-group and of this wave
+    const int wg_last = ((wg_col0 + 128 < ncols) ? wg_col0 + 128 : ncols) - 1;
+    const int khi = start + wg_last / G;
+    int klo = 0;
+    if (window > 0) {
+        klo = start + wg_col0 / G - window + 1;
+        if (klo < 0) klo = 0;
+    }
+    const int t_lo = klo / AT_KEYS, t_hi = khi / AT_KEYS;
+    int wk_lo = 1, wk_hi = 0;                 // empty for a wave without columns
+    if (wave_active) {
+        const int w_last = ((col0 + 32 < ncols) ? col0 + 32 : ncols) - 1;
+        wk_hi = start + w_last / G;
+        wk_lo = 0;
+        if (window > 0) {
+            wk_lo = start + col0 / G - window + 1;
+            if (wk_lo < 0) wk_lo = 0;
+        }
+    }
+    // page ids into LDS
+    {
+        const int32_t* table = tables + (size_t)s * NB;
+        const int npages = (khi >> bs_shift) + 1;
+        for (int i = tid; i < npages; i += 256) tab[i] = table[i];
+    }
 
     uint4 qf[NT][DC];
     int p_col[NT], lo_col[NT], row_col[NT], head_col[NT];
@@ -315,26 +434,6 @@ __global__ __launch_bounds__(256) void attn_mfma_shared_kernel(
         for (int dc = 0; dc < DC; ++dc)
             qf[j][dc] = valid ? *reinterpret_cast<const uint4*>(qp + dc * 32) : make_uint4(0, 0, 0, 0);
     }
-    // key range of the work-group and of this wave, in blocks of 32
-    const int wg_last = ((wg_col0 + 128 < ncols) ? wg_col0 + 128 : ncols) - 1;
-    const int khi = start + wg_last / G;
-    int klo = 0;
-    if (window > 0) {
-        klo = start + wg_col0 / G - window + 1;
-        if (klo < 0) klo = 0;
-    }
-    const int b_lo = klo >> 5, b_hi = khi >> 5;
-    int wb_lo = 1, wb_hi = 0;                 // empty for a wave without columns
-    if (wave_active) {
-        const int w_last = ((col0 + 32 < ncols) ? col0 + 32 : ncols) - 1;
-        wb_hi = (start + w_last / G) >> 5;
-        int wl = 0;
-        if (window > 0) {
-            wl = start + col0 / G - window + 1;
-            if (wl < 0) wl = 0;
-        }
-        wb_lo = wl >> 5;
-    }
 
     float m_run[NT], l_run[NT];
     f32x4 acc[NT][DB];
@@ -346,72 +445,70 @@ __global__ __launch_bounds__(256) void attn_mfma_shared_kernel(
         for (int db = 0; db < DB; ++db) acc[j][db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // loader: thread -> 16-byte units of the K block (key, unit) and of the V^T block (dim, unit)
-    constexpr int KL = (KU + 255) / 256, VL = (VU + 255) / 256;
-    uint4 kreg[KL], vreg[VL];
-    auto fetch = [&](int b) {
-        const int kb = b << 5;
+    // Loader.  A K tile is 64 keys x D/8 units of 16 bytes, a V^T tile D dims x 8 units (8 keys
+    // each): DC units of each per thread.  K: consecutive threads take consecutive units of a key
+    // row.  V^T: consecutive threads take the units of one dim inside a page, then the next dim,
+    // which is how a page lies in memory ([dim][token]); `opp` units of a dim are in one page.
+    const int opp_shift = (bs_shift < 6) ? bs_shift - 3 : 3;    // log2(min(bs, 64) / 8)
+    constexpr int UPK = D / 8;                               // units per key row
+    const int k_key0 = tid / UPK, k_unit = tid % UPK;        // unit i of the thread: key k_key0 + i * 256 / UPK
+    int v_at[DC];                                            // dim | first key of the unit within the tile << 16
 #pragma unroll
-        for (int i = 0; i < KL; ++i) {
-            const int u = tid + 256 * i;
-            int key = kb + u / (D / 8);
-            if (key > khi) key = khi;                        // masked for every column; stay on owned pages
-            const bf16_t* p = kc + ((size_t)(table[key / bs] * bs + key % bs) * nkv + kvh) * D + (u % (D / 8)) * 8;
-            kreg[i] = (u < KU) ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < VL; ++i) {
-            const int u = tid + 256 * i;
-            const int dim = (u >> 2) % D;
-            int vk = kb + (u & 3) * 8;
-            if (vk > khi) vk = khi & ~7;
-            const bf16_t* p = vc + (((size_t)table[vk / bs] * nkv + kvh) * D + dim) * bs + vk % bs;
-            vreg[i] = (u < VU) ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
-        }
-    };
-    auto stash = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < KL; ++i) {
-            const int u = tid + 256 * i;
-            if (u < KU) ks[buf][(u / (D / 8)) * KP + u % (D / 8)] = kreg[i];
-        }
-#pragma unroll
-        for (int i = 0; i < VL; ++i) {
-            const int u = tid + 256 * i;
-            if (u < VU) vs[buf][(u >> 2) * VP + (u & 3)] = vreg[i];
-        }
-    };
-
-    // Three LDS buffers: blocks b and b + 1 are in LDS while block b + 2 is on its way in registers,
-    // so a block's loads have a whole iteration to arrive before they are needed.
-    fetch(b_lo);
-    stash(0);
-    if (b_lo + 1 <= b_hi) {
-        fetch(b_lo + 1);
-        stash(1);
+    for (int i = 0; i < DC; ++i) {
+        const int u = tid + 256 * i;
+        const int o = u & ((1 << opp_shift) - 1);
+        const int rest = u >> opp_shift;
+        v_at[i] = (rest % D) | (((((rest / D) << opp_shift) + o) * 8) << 16);
     }
-    if (b_lo + 2 <= b_hi) fetch(b_lo + 2);
+    uint4 kreg[DC], vreg[DC];
+#define AT_PAGE(KEY, PG, OFF)                                                                                  \
+    OFF = (KEY) & (bs - 1);                                                                                   \
+    PG = tab[(KEY) >> bs_shift];
+#define AT_FETCH(T)                                                                                            \
+    {                                                                                                         \
+        const int kb_ = (T) * AT_KEYS;                                                                        \
+        _Pragma("unroll") for (int i = 0; i < DC; ++i) {                                                      \
+            int key_ = kb_ + k_key0 + i * (256 / UPK);                                                        \
+            if (key_ > khi) key_ = khi; /* masked for every column; stay on owned pages */                    \
+            int pg_, off_;                                                                                    \
+            AT_PAGE(key_, pg_, off_)                                                                          \
+            kreg[i] = *reinterpret_cast<const uint4*>(kc + ((size_t)(pg_ * bs + off_) * nkv + kvh) * D + k_unit * 8); \
+        }                                                                                                     \
+        _Pragma("unroll") for (int i = 0; i < DC; ++i) {                                                      \
+            int vk_ = kb_ + (v_at[i] >> 16);                                                                  \
+            if (vk_ > khi) vk_ = khi & ~7;                                                                    \
+            int pg_, off_;                                                                                    \
+            AT_PAGE(vk_, pg_, off_)                                                                           \
+            vreg[i] = *reinterpret_cast<const uint4*>(vc + (((size_t)pg_ * nkv + kvh) * D + (v_at[i] & 0xffff)) * bs + off_); \
+        }                                                                                                     \
+    }
+#define AT_STASH(BUF)                                                                                          \
+    {                                                                                                         \
+        _Pragma("unroll") for (int i = 0; i < DC; ++i) {                                                      \
+            ks[(BUF) * AT_KEYS * KP + at_lds_row(k_key0 + i * (256 / UPK)) * KP + k_unit] = kreg[i];           \
+            vs[(BUF) * D * VP + (v_at[i] & 0xffff) * VP + (v_at[i] >> 19)] = vreg[i];                          \
+        }                                                                                                     \
+    }
+
+    __syncthreads();                                         // the page ids are in LDS
+    AT_FETCH(t_lo)
+    AT_STASH(0)
     __syncthreads();
-    const int krow0 = 8 * (c >> 2) + (c & 3);                // key of row c in tile 0; tile 1: + 4
     int cur = 0;
-    for (int b = b_lo; b <= b_hi; ++b) {
-        if (b >= wb_lo && b <= wb_hi) {
-            const int kb = b << 5;
-            uint4 kf0[DC], kf1[DC], vf[DB];
+    for (int t = t_lo; t <= t_hi; ++t) {
+        AT_FETCH(t < t_hi ? t + 1 : t)                       // past the last tile: the same again, unused
+        const uint4* kt = ks + cur * AT_KEYS * KP;
+        const uint4* vt = vs + cur * D * VP;
 #pragma unroll
-            for (int dc = 0; dc < DC; ++dc) {
-                kf0[dc] = ks[cur][krow0 * KP + dc * 4 + g];
-                kf1[dc] = ks[cur][(krow0 + 4) * KP + dc * 4 + g];
-            }
-#pragma unroll
-            for (int db = 0; db < DB; ++db) vf[db] = vs[cur][(db * 16 + c) * VP + g];
-            am_block<DC, NT>(kf0, kf1, vf, qf, p_col, lo_col, kb, g, scale2, m_run, l_run, acc);
+        for (int half = 0; half < 2; ++half) {
+            const int kb = t * AT_KEYS + half * 32;
+            if (kb > wk_hi || kb + 31 < wk_lo) continue;      // the same for the whole wave
+            am_block_lds<DC, NT, KP, VP>(kt + half * 32 * KP, vt + half * 4, qf, p_col, lo_col, kb, c, g, scale2, m_run,
+                                         l_run, acc);
         }
-        const int nxt2 = (cur + 2 >= 3) ? cur - 1 : cur + 2;
-        if (b + 2 <= b_hi) stash(nxt2);                      // block b + 2: requested an iteration ago
-        if (b + 3 <= b_hi) fetch(b + 3);
+        AT_STASH(cur ^ 1)
         __syncthreads();
-        cur = (cur + 1 >= 3) ? 0 : cur + 1;
+        cur ^= 1;
     }
 
 #pragma unroll
@@ -430,6 +527,16 @@ __global__ __launch_bounds__(256) void attn_mfma_shared_kernel(
             *reinterpret_cast<uint2*>(op + db * 16) = w;
         }
     }
+}
+
+#undef AT_PAGE
+#undef AT_FETCH
+#undef AT_STASH
+
+// LDS of the tile kernel for head size 32 * DC and a table of `pages` page ids
+static size_t at_lds_bytes(int DC, int pages) {
+    const int D = DC * 32;
+    return (size_t)(2 * AT_KEYS * (D / 8 + 1) + 2 * D * (AT_KEYS / 8 + 1)) * sizeof(uint4) + (size_t)pages * sizeof(int);
 }
 
 // Merge the splits of one (token, head): M = max m_s, out = sum acc_s e^(m_s - M) / sum l_s e^(m_s - M),
@@ -488,8 +595,7 @@ static void launch_attn(int NT, dim3 grid, hipStream_t stream, const bf16_t* q, 
 // blocks of 32 keys, nsplit * split_blocks * 32 must cover the longest context, pos is int32 [T]
 // (the tokens' positions), ws_o holds T*nq*nsplit*d floats and ws_ml T*nq*nsplit*2.  shared != 0
 // runs unsplit steps with prompt portions on the kernel that shares keys and values through LDS
-// (measured slower than independent waves so far: 217 against 177 us for 2,048 tokens at 28/4 heads
-// of 128; kept selectable for tuning).
+// (when the page size and the table length allow it); shared == 0 keeps them on independent waves.
 extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int32_t* tables, int NB, const int32_t* q_start, const int32_t* ctx_start,
                                  const int32_t* pos, void* out, int out_stride, float* ws_o, float* ws_ml, int T, int S,
@@ -514,17 +620,21 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     TL_CHECK_ARG((waves + 3) / 4 <= 65535, "tl_attention_mfma: too many tile groups x splits (%ld)", waves);
     dim3 grid(S, nkv, (unsigned)((waves + 3) / 4));
     const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
-    if (NT == 2 && nsplit == 1 && shared) {
+    const bool pow2 = (bs & (bs - 1)) == 0;
+    if (NT == 2 && nsplit == 1 && shared && pow2 && at_lds_bytes(d / 32, NB) <= 72 * 1024) {
         // 128 columns per work-group, keys and values shared through LDS
+        int bs_shift = 0;
+        while ((1 << bs_shift) < bs) ++bs_shift;
         dim3 sgrid(S, nkv, (unsigned)((max_tile_groups + 3) / 4));
-#define TL_SHARED_CASE(DCV)                                                                                           \
-    hipLaunchKernelGGL((attn_mfma_shared_kernel<DCV>), sgrid, dim3(256), 0, stream, qq, q_stride, kk, vv, tables, NB,   \
-                       q_start, ctx_start, (bf16_t*)out, out_stride, nq, nkv, bs, window, scale)
-        if (d == 32) TL_SHARED_CASE(1);
-        else if (d == 64) TL_SHARED_CASE(2);
-        else TL_SHARED_CASE(4);
-#undef TL_SHARED_CASE
-        TL_CHECK_LAUNCH("tl_attention_mfma shared");
+        const size_t lds = at_lds_bytes(d / 32, NB);
+#define TL_TILE_CASE(DCV)                                                                                             \
+    hipLaunchKernelGGL((attn_tile_kernel<DCV>), sgrid, dim3(256), lds, stream, qq, q_stride, kk, vv, tables, NB,       \
+                       q_start, ctx_start, (bf16_t*)out, out_stride, nq, nkv, bs, bs_shift, window, scale)
+        if (d == 32) TL_TILE_CASE(1);
+        else if (d == 64) TL_TILE_CASE(2);
+        else TL_TILE_CASE(4);
+#undef TL_TILE_CASE
+        TL_CHECK_LAUNCH("tl_attention_mfma tiles");
         return 0;
     }
     if (d == 32)

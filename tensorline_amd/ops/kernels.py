@@ -494,7 +494,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     bfloat16 with a head size of 32, 64 or 128 and pages of a multiple of 8 tokens runs on the
     matrix cores; that kernel works per sequence and needs ``q_start`` [S+1], ``ctx_start`` [S]
     and the host-side ``plan`` (lengths of the step's sequences).  Everything else runs the
-    any-shape kernel.  ``path`` ("mfma", "mfma-shared" or "generic") forces one of them;
+    any-shape kernel.  ``path`` forces one: "generic", "mfma" (prompt portions on the kernel that
+    shares key tiles through LDS where the page size allows) or "mfma-direct" (independent waves);
     ``split_keys`` forces the number of keys per split (0: no split)."""
     _on_gpu(q, k_cache, v_cache, tables, seq_of_token, pos, out, q_start, ctx_start)
     T = q.shape[0]
@@ -512,7 +513,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     mfma_ok = (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and page % 8 == 0 and q_start is not None
                and ctx_start is not None and plan is not None and q_stride % 8 == 0 and o_stride % 4 == 0
                and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0)
-    if path in ("mfma", "mfma-shared"):
+    if path in ("mfma", "mfma-direct"):
         _check(mfma_ok, "paged_attention: the matrix-core kernel does not take these arguments")
     if mfma_ok and path != "generic":
         S = tables.shape[0]
@@ -545,7 +546,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
               _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,
               num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,
-              1 if path == "mfma-shared" else 0, _stream())
+              0 if path == "mfma-direct" else 1, _stream())
         return out
     _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
           _ptr(seq_of_token), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, num_heads,

@@ -348,7 +348,7 @@ def test_attention_portions_and_spike(dtype, nq, nkv, d, bs):
     torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
 
 
-@pytest.mark.parametrize("path", ["generic", "mfma", "mfma-shared"])
+@pytest.mark.parametrize("path", ["generic", "mfma", "mfma-direct"])
 @pytest.mark.parametrize("heads", [(14, 2), (12, 2), (16, 2), (4, 4), (28, 4)])
 @pytest.mark.parametrize("d", [32, 64, 128])
 def test_attention_matrix_core_kernel(path, heads, d):
