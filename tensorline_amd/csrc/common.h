@@ -72,6 +72,24 @@ __device__ __forceinline__ float tl_block_max(float v, float* scratch) {
     return r;
 }
 
+// What a matrix product does for the RMS norms around it (gemm_skinny.hip, gemm_rows64.hip);
+// bfloat16 activations.  Passed by the caller as a pointer (null: nothing).
+struct TlNormArgs {
+    // owed normalisation of A's rows (null: none): ss_in [ss_n, ss_ld] holds ss_n partial sums per
+    // row, row m in column m (a wave reads four partials of all rows from one stretch of memory)
+    const float* ss_in;
+    int ss_ld, ss_n;
+    float dim, eps;            // result rows are scaled by 1/sqrt(sum / dim + eps)
+    // residual add and next norm's input (MODE_PLAIN; null: none)
+    float* resid;              // [M, resid_ld] float, updated in place
+    int resid_ld;
+    const float* next_weight;  // [N]
+    bf16_t* a_out;             // [M, a_ld] = resid * next_weight
+    int a_ld;
+    float* ss_out;             // [tiles, ss_out_ld]: row `tile` gets the tile's sums of resid^2, one per row
+    int ss_out_ld;
+};
+
 // ---- host side -----------------------------------------------------------------------------
 // Every C entry point returns 0 on success.  On failure it returns a non-zero code and leaves a
 // message that tl_last_error() hands out; nothing is launched in that case.

@@ -61,9 +61,11 @@ __device__ __forceinline__ void r64_issue(const bf16_t* const (&xp)[P], const ui
 template <typename TO, int P, int THREADS>
 __global__ __launch_bounds__(THREADS) void gemm_rows64_kernel(
     const bf16_t* __restrict__ A, const uint4* __restrict__ Ws, const float* __restrict__ bias, TO* __restrict__ C,
-    float* __restrict__ partial, int M, int N, int K, int K32, int lda, int ldc, int steps_per_share, int ntiles) {
+    float* __restrict__ partial, int M, int N, int K, int K32, int lda, int ldc, int steps_per_share, int ntiles,
+    TlNormArgs na) {
     constexpr int DEPTH = R64_DEPTH;
     __shared__ uint4 xs[2][R64_MT * R64_UNITS * R64_ROWPAD];
+    __shared__ float sh_rstd[64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nthreads = blockDim.x;
     const int r = lane & 15, g = lane >> 4;
@@ -136,43 +138,108 @@ __global__ __launch_bounds__(THREADS) void gemm_rows64_kernel(
             cur ^= 1;
         }
     }
+    // An owed normalisation is applied here only when the sums are complete (one share): thread
+    // (row, group) adds every ngroups-th partial of its row, one thread per row adds the groups in
+    // order.  The staging buffers are done with and serve as scratch.
+    const bool owed = na.ss_in != nullptr && partial == nullptr;
+    if (owed) {
+        __syncthreads();
+        float* part_sh = reinterpret_cast<float*>(&xs[0][0]);    // [ngroups][64], ngroups <= 16
+        const int row = tid & 63, grp = tid >> 6, ngroups = nthreads >> 6;
+        float ssum = 0.f;
+        if (row < M)
+            for (int t = grp; t < na.ss_n; t += ngroups) ssum += na.ss_in[(size_t)t * na.ss_ld + row];
+        part_sh[grp * 64 + row] = ssum;
+        __syncthreads();
+        if (tid < 64) {
+            float tot = 0.f;
+            for (int g2 = 0; g2 < ngroups; ++g2) tot += part_sh[g2 * 64 + tid];
+            sh_rstd[tid] = 1.0f / sqrtf(tot / na.dim + na.eps);
+        }
+        __syncthreads();
+    }
     if (!tile_live) return;
     // accumulator register i of lane l: C[m = mt*16 + l % 16][n = tile*16 + 4*(l / 16) + i]
     const int n0 = tile * 16 + 4 * g;
+    const bool sink = na.resid != nullptr && partial == nullptr;
 #pragma unroll
     for (int mt = 0; mt < R64_MT; ++mt) {
         const int m = mt * 16 + r;
-        if (m >= M) continue;
+        float sq = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int n = n0 + i;
-            if (n >= N) continue;
+            if (m >= M || n >= N) continue;
             if (partial) {
                 partial[((size_t)blockIdx.y * M + m) * N + n] = acc[mt][i];
-            } else {
-                C[(size_t)m * ldc + n] = tl_from_float<TO>(acc[mt][i] + (bias ? bias[n] : 0.f));
+                continue;
             }
+            float v = owed ? acc[mt][i] * sh_rstd[m] : acc[mt][i];
+            if (bias) v += bias[n];
+            if (sink) {
+                float* rp = na.resid + (size_t)m * na.resid_ld + n;
+                const float h = *rp + v;
+                *rp = h;
+                na.a_out[(size_t)m * na.a_ld + n] = tl_from_float<bf16_t>(h * na.next_weight[n]);
+                sq += h * h;
+            } else {
+                C[(size_t)m * ldc + n] = tl_from_float<TO>(v);
+            }
+        }
+        if (sink) {
+            // the tile's sum of squares of row m: over this lane's four columns, then over the four lanes
+            sq += __shfl_xor(sq, 16, TL_WAVE);
+            sq += __shfl_xor(sq, 32, TL_WAVE);
+            if (g == 0 && m < M) na.ss_out[(size_t)tile * na.ss_out_ld + m] = sq;
         }
     }
 }
 
 // out[m, n] = sum over shares of partial[share, m, n] (+ bias[n]); with swiglu: n < I and
 // out[m, n] = silu(sum gate) * (sum up), gate at column n and up at column I + n of the partials.
+// One group per (256 columns, row).  With an owed normalisation the sums are scaled by the row's
+// 1/sqrt(sum of partials / dim + eps) first; with a residual sink the result is added into the
+// residual, the next norm's input is written and the group's sum of squares becomes one partial.
 template <typename TO>
-__global__ void gemm_rows64_reduce_kernel(const float* __restrict__ partial, const float* __restrict__ bias,
-                                          TO* __restrict__ C, int M, int N, int n_out, int ldc, int shares, int swiglu) {
+__global__ __launch_bounds__(256) void gemm_rows64_reduce_kernel(const float* __restrict__ partial,
+                                                                 const float* __restrict__ bias, TO* __restrict__ C,
+                                                                 int M, int N, int n_out, int ldc, int shares,
+                                                                 int swiglu, TlNormArgs na) {
+    __shared__ float red[16];
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
     const int m = blockIdx.y;
-    if (n >= n_out) return;
-    float v = 0.f, u = 0.f;
-    for (int s = 0; s < shares; ++s) {
-        const float* p = partial + ((size_t)s * M + m) * N;
-        v += p[n];
-        if (swiglu) u += p[n_out + n];
+    float rs = 1.f;
+    if (na.ss_in) {
+        float ssum = 0.f;
+        for (int t = threadIdx.x; t < na.ss_n; t += blockDim.x) ssum += na.ss_in[(size_t)t * na.ss_ld + m];
+        rs = 1.0f / sqrtf(tl_block_sum(ssum, red) / na.dim + na.eps);
     }
-    if (swiglu) v = v / (1.0f + expf(-v)) * u;
-    else if (bias) v += bias[n];
-    C[(size_t)m * ldc + n] = tl_from_float<TO>(v);
+    const bool live = n < n_out;
+    float v = 0.f, u = 0.f;
+    if (live) {
+        for (int s = 0; s < shares; ++s) {
+            const float* p = partial + ((size_t)s * M + m) * N;
+            v += p[n];
+            if (swiglu) u += p[n_out + n];
+        }
+        v *= rs;
+        if (swiglu) v = v / (1.0f + expf(-v)) * (u * rs);
+        else if (bias) v += bias[n];
+    }
+    if (na.resid) {
+        float sq = 0.f;
+        if (live) {
+            float* rp = na.resid + (size_t)m * na.resid_ld + n;
+            const float h = *rp + v;
+            *rp = h;
+            na.a_out[(size_t)m * na.a_ld + n] = tl_from_float<bf16_t>(h * na.next_weight[n]);
+            sq = h * h;
+        }
+        const float tot = tl_block_sum(sq, red);
+        if (threadIdx.x == 0) na.ss_out[(size_t)blockIdx.x * na.ss_out_ld + m] = tot;
+        return;
+    }
+    if (live) C[(size_t)m * ldc + n] = tl_from_float<TO>(v);
 }
 
 // The cut of a [N, K] product with M rows: waves per group and shares of K.  The cost of a cut is
@@ -214,25 +281,29 @@ extern "C" int tl_gemm_rows64_shares(int M, int N, int K) { return r64_plan(M, N
 
 template <typename TO>
 static void r64_launch(const R64Plan& p, hipStream_t stream, const bf16_t* A, const uint4* Ws, const float* bias, TO* C,
-                       float* part, int M, int N, int K, int K32, int lda, int ldc, int ntiles) {
+                       float* part, int M, int N, int K, int K32, int lda, int ldc, int ntiles, const TlNormArgs& na) {
     dim3 grid(p.groups_x, p.shares), block(p.waves * 64);
     if (p.waves >= 16)
         hipLaunchKernelGGL((gemm_rows64_kernel<TO, 1, 1024>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K, K32,
-                           lda, ldc, p.steps, ntiles);
+                           lda, ldc, p.steps, ntiles, na);
     else if (p.waves >= 8)
         hipLaunchKernelGGL((gemm_rows64_kernel<TO, 2, 1024>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K, K32,
-                           lda, ldc, p.steps, ntiles);
+                           lda, ldc, p.steps, ntiles, na);
     else
         hipLaunchKernelGGL((gemm_rows64_kernel<TO, 4, 512>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K, K32,
-                           lda, ldc, p.steps, ntiles);
+                           lda, ldc, p.steps, ntiles, na);
 }
 
 // A: bfloat16 [M, K], 16 < M <= 64 is what it is for (any M from 1 to 64 works); Ws: shuffled copy of
 // W [N, K]; C [M, n_out] bfloat16 or float.  shares = tl_gemm_rows64_shares(M, N, K); with shares > 1
 // `partial` holds shares*M*N floats.  swiglu: W is a fused [2I, K] gate/up matrix (N = 2I), C is
-// [M, I] = silu(gate) * up and bias is not used.
+// [M, I] = silu(gate) * up and bias is not used; it needs shares > 1.  norm: null, or an owed
+// normalisation of A's rows and / or a residual sink (TlNormArgs).  With a sink C is not written,
+// swiglu is not allowed, and ss_out gets one partial per row and 16-column tile when shares is 1
+// ([ceil(N/16), M]), per row and 256 columns otherwise ([ceil(N/256), M]).
 extern "C" int tl_gemm_rows64(const void* A, const void* Ws, const float* bias, void* C, int c_dtype, float* partial,
-                              int M, int N, int K, int lda, int ldc, int shares, int swiglu, hipStream_t stream) {
+                              int M, int N, int K, int lda, int ldc, int shares, int swiglu, const TlNormArgs* norm,
+                              hipStream_t stream) {
     TL_CHECK_ARG(M >= 0 && M <= 64 && N > 0 && K > 0, "tl_gemm_rows64: bad sizes M=%d N=%d K=%d", M, N, K);
     TL_CHECK_ARG(K % 8 == 0 && lda % 8 == 0 && lda >= K, "tl_gemm_rows64: K=%d and the row stride %d must be multiples of 8", K, lda);
     TL_CHECK_ARG(((uintptr_t)A % 16) == 0 && ((uintptr_t)Ws % 16) == 0, "tl_gemm_rows64: operands must be 16-byte aligned");
@@ -241,24 +312,33 @@ extern "C" int tl_gemm_rows64(const void* A, const void* Ws, const float* bias, 
     TL_CHECK_ARG(shares == 1 || partial, "tl_gemm_rows64: shares need a workspace");
     TL_CHECK_ARG(!swiglu || (N % 2 == 0 && shares > 1), "tl_gemm_rows64: the SwiGLU form needs N even and split K");
     const int n_out = swiglu ? N / 2 : N;
-    TL_CHECK_ARG(ldc >= n_out && C, "tl_gemm_rows64: bad output");
+    TlNormArgs na = TlNormArgs();
+    if (norm) na = *norm;
+    if (na.ss_in)
+        TL_CHECK_ARG(na.ss_n > 0 && na.ss_ld >= M && na.dim > 0.f && na.eps >= 0.f,
+                     "tl_gemm_rows64: bad owed-norm arguments (partials %d, stride %d)", na.ss_n, na.ss_ld);
+    if (na.resid)
+        TL_CHECK_ARG(!swiglu && na.next_weight && na.a_out && na.ss_out && na.resid_ld >= N && na.a_ld >= N &&
+                         na.ss_out_ld >= M,
+                     "tl_gemm_rows64: bad residual-sink arguments for M=%d N=%d", M, N);
+    TL_CHECK_ARG(na.resid || (ldc >= n_out && C), "tl_gemm_rows64: bad output");
     TL_CHECK_ARG(c_dtype == TL_F32 || c_dtype == TL_BF16, "tl_gemm_rows64: unknown output dtype %d", c_dtype);
     if (M == 0) return 0;
     const int K32 = tl_ceil_div(K, 32), ntiles = tl_ceil_div(N, 16);
     float* part = shares > 1 ? partial : nullptr;
     if (c_dtype == TL_F32)
-        r64_launch<float>(plan, stream, (const bf16_t*)A, (const uint4*)Ws, bias, (float*)C, part, M, N, K, K32, lda, ldc, ntiles);
+        r64_launch<float>(plan, stream, (const bf16_t*)A, (const uint4*)Ws, bias, (float*)C, part, M, N, K, K32, lda, ldc, ntiles, na);
     else
-        r64_launch<bf16_t>(plan, stream, (const bf16_t*)A, (const uint4*)Ws, bias, (bf16_t*)C, part, M, N, K, K32, lda, ldc, ntiles);
+        r64_launch<bf16_t>(plan, stream, (const bf16_t*)A, (const uint4*)Ws, bias, (bf16_t*)C, part, M, N, K, K32, lda, ldc, ntiles, na);
     TL_CHECK_LAUNCH("tl_gemm_rows64");
     if (shares > 1) {
         dim3 rgrid(tl_ceil_div(n_out, 256), M), rblock(256);
         if (c_dtype == TL_F32)
             hipLaunchKernelGGL(gemm_rows64_reduce_kernel<float>, rgrid, rblock, 0, stream, partial, bias, (float*)C, M, N,
-                               n_out, ldc, shares, swiglu);
+                               n_out, ldc, shares, swiglu, na);
         else
             hipLaunchKernelGGL(gemm_rows64_reduce_kernel<bf16_t>, rgrid, rblock, 0, stream, partial, bias, (bf16_t*)C, M, N,
-                               n_out, ldc, shares, swiglu);
+                               n_out, ldc, shares, swiglu, na);
         TL_CHECK_LAUNCH("tl_gemm_rows64 reduce");
     }
     return 0;

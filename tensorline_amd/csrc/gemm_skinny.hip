@@ -53,21 +53,6 @@ struct QkvArgs {
     int nq, nkv, d, bs;
 };
 
-struct TlNormArgs {
-    // owed normalisation of A's rows (null: none): ss_in [ss_n, ss_ld] holds ss_n partial sums per
-    // row, row m in column m (a wave reads four partials of all rows from one stretch of memory)
-    const float* ss_in;
-    int ss_ld, ss_n;
-    float dim, eps;            // result rows are scaled by 1/sqrt(sum / dim + eps)
-    // residual add and next norm's input (MODE_PLAIN; null: none)
-    float* resid;              // [M, resid_ld] float, updated in place
-    int resid_ld;
-    const float* next_weight;  // [N]
-    bf16_t* a_out;             // [M, a_ld] = resid * next_weight
-    int a_ld;
-    float* ss_out;             // [tiles, ss_out_ld]: row `tile` gets the tile's sums of resid^2, one per row
-    int ss_out_ld;
-};
 
 #define SK_MAX_LDS (80 * 1024)          // LDS of a work-group; a CU has 160 KB
 #define SK_SC 128                    // k values staged per step (4 chunks of 32)

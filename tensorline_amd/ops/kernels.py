@@ -198,12 +198,13 @@ class _NormArgs(ctypes.Structure):
 
 
 def can_defer_norm(num_rows: int, dtype: torch.dtype) -> bool:
-    """Whether the few-row products can carry the norms of a step of ``num_rows`` rows."""
-    return dtype == torch.bfloat16 and 0 < num_rows <= SKINNY_MAX_ROWS
+    """Whether the streaming products can carry the norms of a step of ``num_rows`` rows."""
+    return dtype == torch.bfloat16 and 0 < num_rows <= ROWS64_MAX_ROWS
 
 
-def _norm_args(owed: NormedRows | None, sink: NormSink | None, M: int, N: int, device):
-    """(ctypes argument, NormedRows the sink produces or None) for the few-row entry points."""
+def _norm_args(owed: NormedRows | None, sink: NormSink | None, M: int, N: int, device, columns_per_partial: int = 16):
+    """(ctypes argument, NormedRows the sink produces or None) for the streaming products' entry
+    points; a sink leaves one partial sum of squares per row and ``columns_per_partial`` columns."""
     if owed is None and sink is None:
         return None, None
     na = _NormArgs()
@@ -221,7 +222,7 @@ def _norm_args(owed: NormedRows | None, sink: NormSink | None, M: int, N: int, d
                f"residual sink: the residual must be float32 [{M}, {N}]")
         _check(w.dtype == torch.float32 and w.is_contiguous() and w.numel() == N,
                f"residual sink: the norm weight must be float32 of {N} entries")
-        parts = -(-N // 16)
+        parts = -(-N // columns_per_partial)
         produced = NormedRows(torch.empty(M, N, dtype=torch.bfloat16, device=device),
                               torch.empty(parts, M, dtype=torch.float32, device=device), N, float(sink.eps))
         na.resid, na.resid_ld, na.next_weight = r.data_ptr(), r.stride(0), w.data_ptr()
@@ -253,14 +254,21 @@ def linear(a: torch.Tensor | NormedRows, weight: torch.Tensor, bias: torch.Tenso
     out_dtype = out_dtype or a.dtype
     if owed is not None or sink is not None:
         lda = a.stride(0) if M > 1 else K
-        _check(out is None and _skinny_ok(a, shuffled, M, K, lda),
-               "linear: a deferred norm needs the few-row bfloat16 kernel (at most 16 rows, a shuffled weight copy)")
+        _check(out is None and (_skinny_ok(a, shuffled, M, K, lda) or _rows64_ok(a, shuffled, M, K, lda)),
+               "linear: a deferred norm needs a streaming bfloat16 kernel (at most 64 rows, a shuffled weight copy)")
         _check_shuffled(shuffled, N, K)
-        norm, produced = _norm_args(owed, sink, M, N, a.device)
+        few = M <= SKINNY_MAX_ROWS
+        # a sink's partials: per 16-column tile where the first kernel completes the sums, per 256 columns
+        # where the mid-row product's second kernel does
+        per = 16 if few or library().tl_gemm_rows64_shares(M, N, K) == 1 else 256
+        norm, produced = _norm_args(owed, sink, M, N, a.device, per)
         if produced is None:
             out = torch.empty(M, N, dtype=out_dtype, device=a.device)
-        _call("tl_gemm_skinny", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), F32 if out is None else _code(out, "linear output"),
-              M, N, K, lda, N, norm, _stream())
+        if few:
+            _call("tl_gemm_skinny", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out),
+                  F32 if out is None else _code(out, "linear output"), M, N, K, lda, N, norm, _stream())
+        else:
+            _rows64(a, shuffled, bias, out, M, N, K, lda, N, swiglu=False, norm=norm)
         return produced if produced is not None else out
     if out is None:
         if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and (
@@ -290,12 +298,12 @@ def _rows64_ok(a: torch.Tensor, shuffled: torch.Tensor | None, M: int, K: int, l
             and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0)
 
 
-def _rows64(a, shuffled, bias, out, M, N, K, lda, ldc, swiglu: bool) -> torch.Tensor:
-    """17 to 64 rows: 128 columns per work-group, rows shared through LDS, K split over the grid."""
+def _rows64(a, shuffled, bias, out, M, N, K, lda, ldc, swiglu: bool, norm=None):
+    """17 to 64 rows: a 16-column tile per wave, rows shared through LDS, K split over the grid."""
     shares = library().tl_gemm_rows64_shares(M, N, K)
     ws = torch.empty(shares * M * N, dtype=torch.float32, device=a.device) if shares > 1 else None
-    _call("tl_gemm_rows64", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), _code(out, "linear output"), _ptr(ws),
-          M, N, K, lda, ldc, shares, 1 if swiglu else 0, _stream())
+    _call("tl_gemm_rows64", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), F32 if out is None else _code(out, "linear output"),
+          _ptr(ws), M, N, K, lda, ldc, shares, 1 if swiglu else 0, norm, _stream())
     return out
 
 
@@ -401,13 +409,11 @@ def swiglu_gate_up(h: torch.Tensor | NormedRows, gate_up_weight: torch.Tensor,
         norm, _ = _norm_args(owed, None, M, 2 * I, h.device)
         _call("tl_gemm_skinny_swiglu", _ptr(h), _ptr(shuffled), _ptr(out), M, I, K, lda, I, norm, _stream())
         return out
-    if owed is not None:
-        # the few-row kernel pairs gate and up tiles only for I a multiple of 16: scale the product's rows instead
-        return silu_mul(linear(owed, gate_up_weight, shuffled=shuffled))
     if _rows64_ok(h, shuffled, M, K, lda) and library().tl_gemm_rows64_shares(M, 2 * I, K) > 1:
         out = torch.empty(M, I, dtype=h.dtype, device=h.device)
-        return _rows64(h, shuffled, None, out, M, 2 * I, K, lda, I, swiglu=True)
-    return silu_mul(linear(h, gate_up_weight, shuffled=shuffled))
+        norm, _ = _norm_args(owed, None, M, 2 * I, h.device)
+        return _rows64(h, shuffled, None, out, M, 2 * I, K, lda, I, swiglu=True, norm=norm)
+    return silu_mul(linear(owed if owed is not None else h, gate_up_weight, shuffled=shuffled))
 
 
 def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, who: str) -> None:

@@ -175,7 +175,7 @@ def test_parts_alone(folder_b):
 
 
 def test_decode_steps_hand_norms_to_the_products(folder_b, monkeypatch):
-    """bfloat16 steps of few rows run one norm kernel only (the first layer's first norm): the other
+    """bfloat16 steps of up to 64 rows run one norm kernel only (the first layer's first norm): the other
     norms ride on the products around them.  The logits agree with the same step run with a norm
     kernel for every norm, whether all rows or some are wanted."""
     from tensorline_amd.cache.manager import CacheManager
@@ -191,22 +191,26 @@ def test_decode_steps_hand_norms_to_the_products(folder_b, monkeypatch):
     calls = []
     real = kernels.add_rmsnorm
     monkeypatch.setattr(kernels, "add_rmsnorm", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
-    prompts = helpers.prompts_for("B", [9, 5, 2], seed=4)
-    for i, p in enumerate(prompts):
-        cache.add_request(i)
-        cache.grow(i, len(p))
-    for want_all in (True, False):
-        entries = [StepEntry(i, p, 0, list(range(len(p))) if want_all else [len(p) - 1]) for i, p in enumerate(prompts)]
-        calls.clear()
-        got = runner.step(entries)
-        assert len(calls) == 1
-        with monkeypatch.context() as m:
-            m.setattr(kernels, "can_defer_norm", lambda rows, dtype: False)
+    for lengths in ([9, 5, 2], [30, 21, 9]):                 # 16 rows: the few-row kernels; 60: the mid-row ones
+        prompts = helpers.prompts_for("B", lengths, seed=4)
+        for i, p in enumerate(prompts):
+            cache.add_request(i)
+            cache.grow(i, len(p))
+        for want_all in (True, False):
+            entries = [StepEntry(i, p, 0, list(range(len(p))) if want_all else [len(p) - 1])
+                       for i, p in enumerate(prompts)]
             calls.clear()
-            ref = runner.step(entries)
-            assert len(calls) == 2 * mc.num_hidden_layers + 1
-        torch.testing.assert_close(got, ref, atol=2e-2, rtol=2e-2)
-        assert (got.argmax(-1) == ref.argmax(-1)).float().mean() > 0.8
+            got = runner.step(entries)
+            assert len(calls) == 1
+            with monkeypatch.context() as m:
+                m.setattr(kernels, "can_defer_norm", lambda rows, dtype: False)
+                calls.clear()
+                ref = runner.step(entries)
+                assert len(calls) == 2 * mc.num_hidden_layers + 1
+            torch.testing.assert_close(got, ref, atol=2e-2, rtol=2e-2)
+            assert (got.argmax(-1) == ref.argmax(-1)).float().mean() > 0.8
+        for i in range(len(prompts)):
+            cache.release(i)
 
 
 def test_toy_mixer_with_state_registers_and_steps(tmp_path):

@@ -207,14 +207,16 @@ def _normed_rows(h, gamma, eps, parts):
     return K().NormedRows((h * gamma).to(torch.bfloat16), ss.contiguous(), H, eps)
 
 
-@pytest.mark.parametrize("M", [1, 7, 16])
-@pytest.mark.parametrize("N,Kd,parts", [(176, 64, 4), (1000, 1184, 74), (3584, 3584, 224), (50, 264, 1)])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 40, 64])
+@pytest.mark.parametrize("N,Kd,parts", [(176, 64, 4), (1000, 1184, 74), (3584, 3584, 224), (50, 264, 1), (37888, 3584, 14)])
 def test_products_apply_an_owed_norm(M, N, Kd, parts):
     """A product of rows h * g with the division by rms(h) owed equals the product of RMSNorm(h) * g:
     plain, gate/up with SiLU, and q/k/v with rotation and cache write."""
     torch.manual_seed(M * 1000 + N)
     eps = 1e-5
     h = torch.randn(M, Kd, device=DEV) * torch.logspace(-1, 2, M, device=DEV)[:, None]   # rows of very different size
+    if N > 30000 and M not in (16, 64):
+        pytest.skip("the wide case is for the fullest row counts")
     gamma = 1 + 0.1 * torch.randn(Kd, device=DEV)
     owed = _normed_rows(h, gamma, eps, parts)
     rstd = 1 / torch.sqrt((h.double() ** 2).mean(1, keepdim=True) + eps)
@@ -229,7 +231,7 @@ def test_products_apply_an_owed_norm(M, N, Kd, parts):
         y = x @ w.double().T
         want = torch.nn.functional.silu(y[:, :N // 2]) * y[:, N // 2:]
         torch.testing.assert_close(act.double(), want, atol=2e-2, rtol=2e-2)
-    with pytest.raises(K().KernelError, match="few-row"):
+    with pytest.raises(K().KernelError, match="streaming"):
         K().linear(owed, w, b, out_dtype=torch.float32, shuffled=None)
 
 
@@ -256,8 +258,8 @@ def test_fused_projection_applies_an_owed_norm():
         torch.testing.assert_close(a.float(), c.float(), atol=3e-2, rtol=3e-2)
 
 
-@pytest.mark.parametrize("M", [1, 6, 16])
-@pytest.mark.parametrize("N,Kd", [(176, 64), (1000, 1184), (3584, 18944), (40, 264)])
+@pytest.mark.parametrize("M", [1, 6, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,Kd", [(176, 64), (1000, 1184), (3584, 18944), (40, 264), (5000, 256)])
 def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
     torch.manual_seed(M + N)
     eps = 1e-6
@@ -272,7 +274,7 @@ def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
     torch.testing.assert_close(resid.double(), want, atol=1e-3, rtol=1e-4)
     assert isinstance(nxt, K().NormedRows) and nxt.dim == N and nxt.eps == eps
     torch.testing.assert_close(nxt.rows.float(), (resid * gamma).to(torch.bfloat16).float(), atol=0, rtol=2 ** -7)
-    assert tuple(nxt.sumsq.shape) == (-(-N // 16), M)
+    assert nxt.sumsq.shape[1] == M and nxt.sumsq.shape[0] in (-(-N // 16), -(-N // 256))
     torch.testing.assert_close(nxt.sumsq.double().sum(0), (resid.double() ** 2).sum(1), atol=0, rtol=1e-5)
     # handed on: the next product's result equals that of the norm kernel followed by the product
     w2 = (torch.randn(48, N, device=DEV) / math.sqrt(N)).to(torch.bfloat16)
