@@ -52,6 +52,7 @@ class _Request:
     state_slot: int
     hashes: list[int] = field(default_factory=list)   # content hashes of its full, computed pages
     arrays: list = field(default_factory=list)        # per group: the table as an int32 array, or None when stale
+    serial: int = 0                                   # which admission of the request this is (never reused)
 
 
 class CacheManager:
@@ -89,6 +90,8 @@ class CacheManager:
             self.groups[g].entries.append(i)
             self.group_of_entry[i] = g
             self.storage_entry[i] = i
+        self._windowed = any(g.window > 0 for g in self.groups)
+        self._serial = 0
         # an entry that reads a windowed entry's cache with a wider view would see freed pages
         for i, e in enumerate(schedule):
             if e.cache_from is not None and cache_needs[i] is not None:
@@ -177,9 +180,15 @@ class CacheManager:
         slot = self._free_slots.pop()
         for t in self.state.values():
             t[slot].zero_()
+        self._serial += 1
         self._requests[rid] = _Request([[] for _ in self.groups], [0] * len(self.groups), slot,
-                                       arrays=[None] * len(self.groups))
+                                       arrays=[None] * len(self.groups), serial=self._serial)
         return slot
+
+    def admission(self, rid) -> int:
+        """A number that differs between two admissions of a request id (its pages were given back
+        in between): whoever keeps a copy of a table can tell that it is stale."""
+        return self._requests[rid].serial
 
     def state_slot(self, rid) -> int:
         return self._requests[rid].state_slot
@@ -201,6 +210,8 @@ class CacheManager:
         (reference ``_grow``: tensorline/batch_engine.py:251-259)."""
         req = self._requests[rid]
         want = self.pages_for(upto)
+        if all(len(t) >= want for t in req.tables):          # the usual case of a decoded token: nothing to add
+            return True
         needs = [max(0, want - len(t)) for t in req.tables]
         if any(n > g.allocator.num_free for n, g in zip(needs, self.groups)):
             return False
@@ -216,6 +227,8 @@ class CacheManager:
         """After ``computed`` tokens are cached: give back the pages of windowed groups that hold
         only positions no later token can see.  The next token sits at position ``computed`` and
         sees keys from ``computed - window + 1`` on.  Returns the number of pages given back."""
+        if not self._windowed:
+            return 0
         req = self._requests[rid]
         given = 0
         for gi, g in enumerate(self.groups):

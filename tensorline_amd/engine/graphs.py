@@ -20,6 +20,7 @@ from __future__ import annotations
 
 from typing import Sequence
 
+import numpy as np
 import torch
 
 from tensorline_amd.cache.manager import CacheManager
@@ -38,6 +39,11 @@ def _pow2_upto(limit: int) -> list[int]:
 class _Captured:
     def __init__(self, graph, dev, host, logits, packed):
         self.graph, self.dev, self.host, self.logits, self.packed = graph, dev, host, logits, packed
+        # what the host buffer holds since the last replay: the requests of its rows and their
+        # positions, so that the next token of the same requests only touches a few numbers
+        self.rids: tuple | None = None
+        self.admissions: tuple = ()
+        self.starts: np.ndarray | None = None
 
 
 class GraphRunner(ModelRunner):
@@ -119,6 +125,49 @@ class GraphRunner(ModelRunner):
         torch.cuda.synchronize()
         return len(self.graphs)
 
+    def _advance(self, cap: _Captured, entries: Sequence[StepEntry]) -> bool:
+        """The common case of steady decoding: the same requests in the same rows as the bucket's
+        last replay, each one token further.  Then the buffer is brought up to date in place (token,
+        position, cache row, and a page id where a request entered a new page) instead of being
+        packed again.  False: not that case, nothing was touched."""
+        cache = self.cache
+        if cap.rids is None or len(cap.rids) != len(entries) or cache._windowed:
+            return False
+        for rid, adm, e in zip(cap.rids, cap.admissions, entries):
+            if e.rid != rid or cache.admission(rid) != adm:  # another request, or the same one admitted again
+                return False
+        n = len(entries)
+        starts = np.fromiter((e.start for e in entries), np.int64, n)
+        if not np.array_equal(starts, cap.starts + 1):
+            return False
+        toks = np.fromiter((e.tokens[0] for e in entries), np.int64, n)
+        if toks.min() < 0 or toks.max() >= self.model.vocab_size:
+            raise ValueError(f"token id outside [0, {self.model.vocab_size})")
+        buf, off = cap.host.numpy(), cap.packed.offsets
+        page = cache.page_size
+        lp, within = starts // page, starts % page
+        fresh = np.nonzero(within == 0)[0]                   # requests whose token opens a page
+        rows = np.arange(n)
+        for g in range(len(cache.groups)):
+            o, size = off[f"tables{g}"]
+            tables = buf[o:o + size].reshape(cap.packed.S, cap.packed.group_nb[g])
+            for i in fresh:
+                tab = cache.table_array(cap.rids[i], g)
+                if len(tab) <= lp[i]:
+                    raise ValueError(f"request {cap.rids[i]!r}: page table covers {len(tab) * page} tokens, "
+                                     f"{starts[i] + 1} are needed")
+                tables[i, lp[i]] = tab[lp[i]]
+            pages = tables[rows, lp]
+            if pages.min() < 0:
+                raise ValueError("a token of this step lies on a page already given back")
+            o, _ = off[f"slots{g}"]
+            buf[o:o + n] = pages * page + within
+        for name, vals in (("ids", toks), ("pos", starts), ("ctx_start", starts)):
+            o, _ = off[name]
+            buf[o:o + n] = vals
+        cap.starts = starts
+        return True
+
     # ---- one step ------------------------------------------------------------------------------
     @torch.inference_mode()
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -128,9 +177,13 @@ class GraphRunner(ModelRunner):
         B = self._bucket(n)
         cap = self.graphs.get(B) or self._capture(B)
         ng = len(self.cache.groups)
-        packed = self.pack(entries, pad_seqs=B, pad_nb=[self.max_blocks] * ng)
-        assert packed.offsets == cap.packed.offsets, "graph buffer layout changed"
-        cap.host.numpy()[:] = packed.data
+        if not self._advance(cap, entries):
+            packed = self.pack(entries, pad_seqs=B, pad_nb=[self.max_blocks] * ng)
+            assert packed.offsets == cap.packed.offsets, "graph buffer layout changed"
+            cap.host.numpy()[:] = packed.data
+            cap.rids = tuple(e.rid for e in entries)
+            cap.admissions = tuple(self.cache.admission(rid) for rid in cap.rids)
+            cap.starts = np.fromiter((e.start for e in entries), np.int64, n)
         cap.dev.copy_(cap.host, non_blocking=False)
         cap.graph.replay()
         self.graph_replays += 1

@@ -116,8 +116,9 @@ class Scheduler:
     def schedule(self) -> list[tuple[Request, int]]:
         budget = self.max_batched_tokens
         plan: list[tuple[Request, int]] = []
+        preempted: set[int] = set()
         for req in list(self.running):                       # oldest first
-            if req not in self.running:                      # preempted earlier in this pass
+            if id(req) in preempted:                         # preempted earlier in this pass
                 continue
             n = min(len(req.tokens) - req.num_computed, budget)
             if n <= 0:
@@ -126,6 +127,7 @@ class Scheduler:
             while not self.cache.grow(req.rid, req.num_computed + n):
                 victim = self.running[-1]                    # the newest running request
                 self._preempt(victim)
+                preempted.add(id(victim))
                 budget += sum(k for r, k in plan if r is victim)
                 plan = [(r, k) for r, k in plan if r is not victim]
                 if victim is req:

@@ -1,0 +1,85 @@
+"""The replayed decode step's host buffer: bringing it up to date in place gives what packing the
+step again gives, and is not done when it would be wrong (host data only, no GPU)."""
+import numpy as np
+import pytest
+import torch
+
+from tensorline_amd.cache.manager import CacheManager
+from tensorline_amd.engine.batch import StepEntry
+from tensorline_amd.engine.graphs import GraphRunner, _Captured
+from tensorline_amd.parts.spec import CacheNeed, ScheduleEntry
+
+
+class _Model:
+    vocab_size = 1000
+    device = "cpu"
+    schedule = [ScheduleEntry(0)]
+
+
+def _setup(window=0, page=4, max_blocks=8):
+    cache = CacheManager([CacheNeed(1, 8, window)], [ScheduleEntry(0)], [None], page_size=page, num_blocks=40,
+                         max_requests=4, dtype=torch.float32, device="cpu", allocate_storage=False)
+    runner = GraphRunner(_Model(), cache, max_batch=4, max_blocks_per_seq=max_blocks)
+    return cache, runner
+
+
+def _cap(runner, entries, B=4):
+    packed = runner.pack(entries, pad_seqs=B, pad_nb=[runner.max_blocks])
+    host = torch.from_numpy(packed.data.copy())
+    cap = _Captured(None, None, host, None, packed)
+    cap.rids = tuple(e.rid for e in entries)
+    cap.admissions = tuple(runner.cache.admission(r) for r in cap.rids)
+    cap.starts = np.array([e.start for e in entries], np.int64)
+    return cap
+
+
+def test_in_place_update_equals_packing_again():
+    cache, runner = _setup()
+    lens = {"a": 3, "b": 7, "c": 4}
+    for rid, n in lens.items():
+        cache.add_request(rid)
+        assert cache.grow(rid, n + 1)
+    entries = [StepEntry(rid, [5], n, [0]) for rid, n in lens.items()]
+    cap = _cap(runner, entries)
+    rng = np.random.default_rng(0)
+    for step in range(1, 14):                                 # crosses several page boundaries
+        entries = []
+        for rid in lens:
+            lens[rid] += 1
+            assert cache.grow(rid, lens[rid] + 1)
+            entries.append(StepEntry(rid, [int(rng.integers(0, 1000))], lens[rid], [0]))
+        assert runner._advance(cap, entries)
+        want = runner.pack(entries, pad_seqs=4, pad_nb=[runner.max_blocks]).data
+        np.testing.assert_array_equal(cap.host.numpy(), want)
+
+
+def test_in_place_update_declines_when_the_buffer_is_stale():
+    cache, runner = _setup()
+    for rid in "ab":
+        cache.add_request(rid)
+        cache.grow(rid, 6)
+    entries = [StepEntry("a", [1], 5, [0]), StepEntry("b", [2], 5, [0])]
+    cap = _cap(runner, entries)
+    before = cap.host.numpy().copy()
+    nxt = [StepEntry("a", [1], 6, [0]), StepEntry("b", [2], 6, [0])]
+    cache.grow("a", 7), cache.grow("b", 7)
+    assert not runner._advance(cap, nxt[::-1])                # other order of rows
+    assert not runner._advance(cap, nxt[:1])                  # fewer requests
+    assert not runner._advance(cap, [StepEntry("a", [1], 7, [0]), nxt[1]])   # a request moved two tokens
+    cache.release("a")                                        # given back and admitted again: other pages
+    cache.add_request("a")
+    cache.grow("a", 7)
+    assert not runner._advance(cap, nxt)
+    np.testing.assert_array_equal(cap.host.numpy(), before)   # declining touches nothing
+    with pytest.raises(ValueError, match="token id"):
+        cap2 = _cap(runner, entries)
+        runner._advance(cap2, [StepEntry("a", [1000], 6, [0]), nxt[1]])
+
+
+def test_in_place_update_is_off_for_windowed_caches():
+    cache, runner = _setup(window=6)
+    cache.add_request("a")
+    cache.grow("a", 6)
+    cap = _cap(runner, [StepEntry("a", [1], 5, [0])])
+    cache.grow("a", 7)
+    assert not runner._advance(cap, [StepEntry("a", [1], 6, [0])])
