@@ -242,6 +242,64 @@ __global__ __launch_bounds__(256) void gemm_rows64_reduce_kernel(const float* __
     if (live) C[(size_t)m * ldc + n] = tl_from_float<TO>(v);
 }
 
+// The second kernel of a fused q/k/v projection: sums of the shares (scaled by an owed
+// normalisation), bias, rotate-half RoPE of query and key heads by the token's position (angle
+// pos * inv_freq[i] in float, as tl_rope_store does), queries to q_out [M, nq*d], rotated keys and
+// the values into the paged cache at slots[m] (k_cache [pages, page, nkv, d], v_cache
+// [pages, nkv, d, page]; a negative slot stores nothing).  One thread per (row, head, pair of dims
+// idx and idx + d/2); full-width rotation only.
+__global__ __launch_bounds__(256) void gemm_rows64_reduce_qkv_kernel(
+    const float* __restrict__ partial, const float* __restrict__ bias, int M, int N, int shares,
+    const int32_t* __restrict__ pos, const float* __restrict__ inv_freq, const int32_t* __restrict__ slots,
+    bf16_t* __restrict__ q_out, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int nq, int nkv, int d,
+    int bs, TlNormArgs na) {
+    __shared__ float red[16];
+    const int pi = blockIdx.x * blockDim.x + threadIdx.x;
+    const int m = blockIdx.y;
+    float rs = 1.f;
+    if (na.ss_in) {
+        float ssum = 0.f;
+        for (int t = threadIdx.x; t < na.ss_n; t += blockDim.x) ssum += na.ss_in[(size_t)t * na.ss_ld + m];
+        rs = 1.0f / sqrtf(tl_block_sum(ssum, red) / na.dim + na.eps);
+    }
+    const int half = d / 2;
+    if (pi >= N / 2) return;
+    const int head = pi / half, idx = pi - head * half;
+    const int n1 = head * d + idx, n2 = n1 + half;
+    float v = 0.f, u = 0.f;
+    for (int s = 0; s < shares; ++s) {
+        const float* p = partial + ((size_t)s * M + m) * N;
+        v += p[n1];
+        u += p[n2];
+    }
+    v *= rs;
+    u *= rs;
+    if (bias) {
+        v += bias[n1];
+        u += bias[n2];
+    }
+    const int slot = slots[m];
+    if (head < nq + nkv) {
+        float sn, cs;
+        sincosf((float)pos[m] * inv_freq[idx], &sn, &cs);
+        const float o1 = v * cs - u * sn, o2 = u * cs + v * sn;
+        if (head < nq) {
+            bf16_t* qp = q_out + (size_t)m * nq * d + (size_t)head * d + idx;
+            qp[0] = tl_from_float<bf16_t>(o1);
+            qp[half] = tl_from_float<bf16_t>(o2);
+        } else if (slot >= 0) {
+            bf16_t* kp = k_cache + ((size_t)slot * nkv + (head - nq)) * d + idx;
+            kp[0] = tl_from_float<bf16_t>(o1);
+            kp[half] = tl_from_float<bf16_t>(o2);
+        }
+    } else if (slot >= 0) {
+        const int page = slot / bs, off = slot - page * bs;
+        bf16_t* vp = v_cache + (((size_t)page * nkv + (head - nq - nkv)) * d + idx) * bs + off;
+        vp[0] = tl_from_float<bf16_t>(v);
+        vp[(size_t)half * bs] = tl_from_float<bf16_t>(u);
+    }
+}
+
 // The cut of a [N, K] product with M rows: waves per group and shares of K.  The cost of a cut is
 // the work of the busiest CU in units of one wave's step (4 KB of W): whole rounds of groups over
 // the CUs, each group as slow as its waves are many, plus two steps of filling and draining per
@@ -341,5 +399,39 @@ extern "C" int tl_gemm_rows64(const void* A, const void* Ws, const float* bias, 
                                n_out, ldc, shares, swiglu, na);
         TL_CHECK_LAUNCH("tl_gemm_rows64 reduce");
     }
+    return 0;
+}
+
+// The fused q/k/v projection for 17 to 64 rows: the product above with K cut into shares, then
+// gemm_rows64_reduce_qkv_kernel.  Ws is the shuffled copy of the [(nq + 2 nkv) d, K] matrix; shares
+// = tl_gemm_rows64_shares(M, N, K) must be above 1 (the caller uses the separate kernels otherwise)
+// and `partial` holds shares*M*N floats.  norm: null or an owed normalisation of A's rows.
+extern "C" int tl_gemm_rows64_qkv_rope(const void* A, const void* Ws, const float* bias, const int32_t* pos,
+                                       const float* inv_freq, const int32_t* slots, void* q_out, void* k_cache,
+                                       void* v_cache, float* partial, int M, int K, int lda, int nq, int nkv, int d,
+                                       int bs, int shares, const TlNormArgs* norm, hipStream_t stream) {
+    TL_CHECK_ARG(nq > 0 && nkv > 0 && d > 0 && d % 2 == 0 && bs > 0, "tl_gemm_rows64_qkv_rope: bad sizes d=%d nq=%d nkv=%d page=%d", d, nq, nkv, bs);
+    const int N = (nq + 2 * nkv) * d;
+    TL_CHECK_ARG(M >= 0 && M <= 64 && K > 0, "tl_gemm_rows64_qkv_rope: bad sizes M=%d K=%d", M, K);
+    TL_CHECK_ARG(K % 8 == 0 && lda % 8 == 0 && lda >= K, "tl_gemm_rows64_qkv_rope: K=%d and the row stride %d must be multiples of 8", K, lda);
+    TL_CHECK_ARG(((uintptr_t)A % 16) == 0 && ((uintptr_t)Ws % 16) == 0, "tl_gemm_rows64_qkv_rope: operands must be 16-byte aligned");
+    TL_CHECK_ARG(pos && inv_freq && slots && q_out && k_cache && v_cache && partial, "tl_gemm_rows64_qkv_rope: missing argument");
+    const R64Plan plan = r64_plan(M, N, K);
+    TL_CHECK_ARG(shares == plan.shares && shares > 1, "tl_gemm_rows64_qkv_rope: %d shares do not fit this shape, or K is not cut", shares);
+    TlNormArgs na = TlNormArgs();
+    if (norm) na = *norm;
+    TL_CHECK_ARG(!na.resid, "tl_gemm_rows64_qkv_rope: a projection into the cache has no residual sink");
+    if (na.ss_in)
+        TL_CHECK_ARG(na.ss_n > 0 && na.ss_ld >= M && na.dim > 0.f && na.eps >= 0.f,
+                     "tl_gemm_rows64_qkv_rope: bad owed-norm arguments (partials %d, stride %d)", na.ss_n, na.ss_ld);
+    if (M == 0) return 0;
+    const int K32 = tl_ceil_div(K, 32), ntiles = tl_ceil_div(N, 16);
+    r64_launch<bf16_t>(plan, stream, (const bf16_t*)A, (const uint4*)Ws, nullptr, (bf16_t*)nullptr, partial, M, N, K, K32,
+                       lda, N, ntiles, TlNormArgs());
+    TL_CHECK_LAUNCH("tl_gemm_rows64_qkv_rope");
+    dim3 rgrid(tl_ceil_div(N / 2, 256), M), rblock(256);
+    hipLaunchKernelGGL(gemm_rows64_reduce_qkv_kernel, rgrid, rblock, 0, stream, partial, bias, M, N, shares, pos, inv_freq,
+                       slots, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nq, nkv, d, bs, na);
+    TL_CHECK_LAUNCH("tl_gemm_rows64_qkv_rope second kernel");
     return 0;
 }

@@ -433,17 +433,23 @@ def qkv_rope_store(h: torch.Tensor | NormedRows, shuffled: torch.Tensor, bias: t
     """The projection, position encoding and cache write of a decode step in one kernel: returns the
     rotated queries [M, nq*d]; rotated keys and the values go into the cache at ``slots``.  Returns
     None when the kernel does not take the case (then the three separate kernels run): it needs
-    bfloat16, at most 16 rows, a head size that is a multiple of 32 and full-width rotation.
+    bfloat16, at most 64 rows (above 16: a K long enough to be cut into shares), a head size that is
+    a multiple of 32 and full-width rotation.
     ``h`` may be :class:`NormedRows`."""
     owed = h if isinstance(h, NormedRows) else None
     if owed is not None:
         h = owed.rows
     M, K = h.shape
     N = (num_heads + 2 * num_kv_heads) * head_dim
-    if not (h.dtype == torch.bfloat16 and shuffled is not None and M <= 16 and head_dim % 32 == 0
+    if not (h.dtype == torch.bfloat16 and shuffled is not None and M <= ROWS64_MAX_ROWS and head_dim % 32 == 0
             and inv_freq is not None and 2 * inv_freq.numel() == head_dim and h.stride(1) == 1
             and K % 8 == 0 and h.data_ptr() % 16 == 0 and (M == 1 or h.stride(0) % 8 == 0)):
         return None
+    shares = 1
+    if M > SKINNY_MAX_ROWS:
+        shares = library().tl_gemm_rows64_shares(M, N, K)
+        if shares == 1:                                   # the mid-row product fuses only in its second kernel
+            return None
     _on_gpu(h, shuffled, bias, pos, inv_freq, k_cache, v_cache, slots)
     _check_shuffled(shuffled, N, K)
     _check_caches(k_cache, v_cache, h.dtype, num_kv_heads, head_dim, "qkv_rope_store")
@@ -454,6 +460,12 @@ def qkv_rope_store(h: torch.Tensor | NormedRows, shuffled: torch.Tensor, bias: t
         _check(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == N, "qkv_rope_store: bad bias")
     q = torch.empty(M, num_heads * head_dim, dtype=h.dtype, device=h.device)
     norm, _ = _norm_args(owed, None, M, N, h.device)
+    if M > SKINNY_MAX_ROWS:
+        ws = torch.empty(shares * M * N, dtype=torch.float32, device=h.device)
+        _call("tl_gemm_rows64_qkv_rope", _ptr(h), _ptr(shuffled), _ptr(bias), _ptr(pos), _ptr(inv_freq), _ptr(slots),
+              _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(ws), M, K, h.stride(0), num_heads, num_kv_heads, head_dim,
+              k_cache.shape[1], shares, norm, _stream())
+        return q
     _call("tl_gemm_skinny_qkv_rope", _ptr(h), _ptr(shuffled), _ptr(bias), _ptr(pos), _ptr(inv_freq), _ptr(slots),
           _ptr(q), _ptr(k_cache), _ptr(v_cache), M, K, h.stride(0) if M > 1 else K, num_heads, num_kv_heads,
           head_dim, k_cache.shape[1], norm, _stream())
