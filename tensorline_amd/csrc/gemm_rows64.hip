@@ -41,9 +41,10 @@ __device__ __forceinline__ bf16x8 r64_frag(uint4 v) { return __builtin_bit_cast(
 // Loads of one step: this thread's P pieces of A and this lane's four W fragments.  Steps are
 // clamped by the caller, so every address is valid; nothing here depends on the loaded data, so
 // the loads stay in flight until the step that uses them.
-template <int P>
-__device__ __forceinline__ void r64_issue(const bf16_t* const (&xp)[P], const uint4* w1, int step, int xunit, int K,
-                                          int last_c, uint4 (&xo)[P], uint4 (&wo)[4]) {
+template <int P, bool PAIR>
+__device__ __forceinline__ void r64_issue(const bf16_t* const (&xp)[P], const uint4* w1, const uint4* w2, int step,
+                                          int xunit, int K, int last_c, uint4 (&xo)[P], uint4 (&wo)[4],
+                                          uint4 (&uo)[PAIR ? 4 : 1]) {
     const int kbase = (step * R64_SC + xunit * 8 < K) ? step * R64_SC : 0;
 #pragma unroll
     for (int i = 0; i < P; ++i) xo[i] = *reinterpret_cast<const uint4*>(xp[i] + kbase);
@@ -52,13 +53,16 @@ __device__ __forceinline__ void r64_issue(const bf16_t* const (&xp)[P], const ui
         int c = step * 4 + i;
         if (c > last_c) c = last_c;
         wo[i] = w1[(size_t)c * 64];
+        if (PAIR) uo[i] = w2[(size_t)c * 64];
     }
 }
 
 // P: pieces of A a thread loads per step; the group has at least 1024 / P threads (a multiple of
 // 16, so that a thread's pieces all lie in one 16-byte column of the step).  Wave w of group x owns
-// tile w * gridDim.x + x: groups differ by at most one live wave.
-template <typename TO, int P, int THREADS>
+// tile w * gridDim.x + x: groups differ by at most one live wave.  PAIR: W is a fused gate/up
+// matrix of ntiles + ntiles tiles, a wave owns gate tile t and up tile ntiles + t and writes
+// silu(gate) * up to C [M, N / 2] (one share only: the sums must be complete).
+template <typename TO, int P, int THREADS, bool PAIR>
 __global__ __launch_bounds__(THREADS) void gemm_rows64_kernel(
     const bf16_t* __restrict__ A, const uint4* __restrict__ Ws, const float* __restrict__ bias, TO* __restrict__ C,
     float* __restrict__ partial, int M, int N, int K, int K32, int lda, int ldc, int steps_per_share, int ntiles,
@@ -76,12 +80,15 @@ __global__ __launch_bounds__(THREADS) void gemm_rows64_kernel(
     const bool tile_live = tile < ntiles;
     if (!tile_live) tile = ntiles - 1;                       // loads stay in bounds; nothing is written
     const uint4* w1 = Ws + (size_t)tile * K32 * 64 + lane;
+    const uint4* w2 = PAIR ? Ws + (size_t)(ntiles + tile) * K32 * 64 + lane : nullptr;
     const uint4 zero = make_uint4(0, 0, 0, 0);
     const int last_c = K32 - 1;
 
-    f32x4 acc[R64_MT];
+    f32x4 acc[R64_MT], acc2[PAIR ? R64_MT : 1];
 #pragma unroll
     for (int i = 0; i < R64_MT; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < (PAIR ? R64_MT : 1); ++i) acc2[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // loader of A: 64 rows x 16 units = 1024 16-byte pieces, up to P per thread
     const bf16_t* xp[P];
@@ -97,11 +104,11 @@ __global__ __launch_bounds__(THREADS) void gemm_rows64_kernel(
     }
     const int xunit = tid & 15;
     const int nst = s1 - s0;
-    uint4 xa[DEPTH][P], wr[DEPTH][4];
+    uint4 xa[DEPTH][P], wr[DEPTH][4], ur[DEPTH][PAIR ? 4 : 1];
 #pragma unroll
     for (int j = 0; j < DEPTH; ++j) {
         const int st = (j < nst) ? s0 + j : s1 - 1;
-        r64_issue<P>(xp, w1, st, xunit, K, last_c, xa[j], wr[j]);
+        r64_issue<P, PAIR>(xp, w1, w2, st, xunit, K, last_c, xa[j], wr[j], ur[j]);
         __builtin_amdgcn_sched_barrier(0);                   // oldest slot first, as in the loop below
     }
     int cur = 0;
@@ -127,13 +134,15 @@ __global__ __launch_bounds__(THREADS) void gemm_rows64_kernel(
                 for (int mt = 0; mt < R64_MT; ++mt) {
                     const uint4 xf = xs[cur][(mt * R64_UNITS + cc * 4 + g) * R64_ROWPAD + r];
                     acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(r64_frag(wr[j][cc]), r64_frag(xf), acc[mt], 0, 0, 0);
+                    if (PAIR)
+                        acc2[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(r64_frag(ur[j][cc]), r64_frag(xf), acc2[mt], 0, 0, 0);
                 }
             }
             // Refill this slot of the ring only now that its values are used up, so that the slot
             // keeps its registers over the whole loop and nothing has to wait for a copy.
             __builtin_amdgcn_sched_barrier(0);
             const int sn = (it + DEPTH < nst) ? s0 + it + DEPTH : s1 - 1;   // past the end: a step again, unused
-            r64_issue<P>(xp, w1, sn, xunit, K, last_c, xa[j], wr[j]);
+            r64_issue<P, PAIR>(xp, w1, w2, sn, xunit, K, last_c, xa[j], wr[j], ur[j]);
             __builtin_amdgcn_sched_barrier(0);
             cur ^= 1;
         }
@@ -169,12 +178,17 @@ __global__ __launch_bounds__(THREADS) void gemm_rows64_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int n = n0 + i;
-            if (m >= M || n >= N) continue;
+            if (m >= M || n >= (PAIR ? N / 2 : N)) continue;
             if (partial) {
                 partial[((size_t)blockIdx.y * M + m) * N + n] = acc[mt][i];
                 continue;
             }
             float v = owed ? acc[mt][i] * sh_rstd[m] : acc[mt][i];
+            if (PAIR) {
+                const float u = owed ? acc2[mt][i] * sh_rstd[m] : acc2[mt][i];
+                C[(size_t)m * ldc + n] = tl_from_float<TO>(v / (1.0f + expf(-v)) * u);
+                continue;
+            }
             if (bias) v += bias[n];
             if (sink) {
                 float* rp = na.resid + (size_t)m * na.resid_ld + n;
@@ -334,6 +348,24 @@ static R64Plan r64_plan(int M, int N, int K) {
     return best;
 }
 
+// The cut for the paired gate/up form: one share, a wave per pair of tiles (it streams two tiles),
+// at most 7 waves so that a thread's registers hold two rings of fragments.
+static R64Plan r64_plan_pairs(int M, int npairs, int K) {
+    const int nsc = tl_ceil_div(tl_ceil_div(K, 32), 4);
+    R64Plan best{R64_MIN_WAVES, 1, nsc, tl_ceil_div(npairs, R64_MIN_WAVES)};
+    double best_cost = 1e30;
+    for (int waves = R64_MIN_WAVES; waves <= 7; ++waves) {
+        const int gx = tl_ceil_div(npairs, waves);
+        const int live = tl_ceil_div(npairs, gx);
+        const double cost = (double)tl_ceil_div(gx, R64_CUS) * (2 * live + R64_A_WEIGHT) * (nsc + 2);
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = R64Plan{waves, 1, nsc, gx};
+        }
+    }
+    return best;
+}
+
 // Number of shares K is cut into for a [N, K] matrix and M rows (the caller sizes the workspace by it).
 extern "C" int tl_gemm_rows64_shares(int M, int N, int K) { return r64_plan(M, N, K).shares; }
 
@@ -342,20 +374,20 @@ static void r64_launch(const R64Plan& p, hipStream_t stream, const bf16_t* A, co
                        float* part, int M, int N, int K, int K32, int lda, int ldc, int ntiles, const TlNormArgs& na) {
     dim3 grid(p.groups_x, p.shares), block(p.waves * 64);
     if (p.waves >= 16)
-        hipLaunchKernelGGL((gemm_rows64_kernel<TO, 1, 1024>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K, K32,
-                           lda, ldc, p.steps, ntiles, na);
+        hipLaunchKernelGGL((gemm_rows64_kernel<TO, 1, 1024, false>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K,
+                           K32, lda, ldc, p.steps, ntiles, na);
     else if (p.waves >= 8)
-        hipLaunchKernelGGL((gemm_rows64_kernel<TO, 2, 1024>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K, K32,
-                           lda, ldc, p.steps, ntiles, na);
+        hipLaunchKernelGGL((gemm_rows64_kernel<TO, 2, 1024, false>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K,
+                           K32, lda, ldc, p.steps, ntiles, na);
     else
-        hipLaunchKernelGGL((gemm_rows64_kernel<TO, 4, 512>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K, K32,
-                           lda, ldc, p.steps, ntiles, na);
+        hipLaunchKernelGGL((gemm_rows64_kernel<TO, 4, 512, false>), grid, block, 0, stream, A, Ws, bias, C, part, M, N, K,
+                           K32, lda, ldc, p.steps, ntiles, na);
 }
 
 // A: bfloat16 [M, K], 16 < M <= 64 is what it is for (any M from 1 to 64 works); Ws: shuffled copy of
 // W [N, K]; C [M, n_out] bfloat16 or float.  shares = tl_gemm_rows64_shares(M, N, K); with shares > 1
 // `partial` holds shares*M*N floats.  swiglu: W is a fused [2I, K] gate/up matrix (N = 2I), C is
-// [M, I] = silu(gate) * up and bias is not used; it needs shares > 1.  norm: null, or an owed
+// [M, I] = silu(gate) * up and bias is not used (with one share I must be a multiple of 16).  norm: null, or an owed
 // normalisation of A's rows and / or a residual sink (TlNormArgs).  With a sink C is not written,
 // swiglu is not allowed, and ss_out gets one partial per row and 16-column tile when shares is 1
 // ([ceil(N/16), M]), per row and 256 columns otherwise ([ceil(N/256), M]).
@@ -368,7 +400,8 @@ extern "C" int tl_gemm_rows64(const void* A, const void* Ws, const float* bias, 
     const R64Plan plan = r64_plan(M, N, K);
     TL_CHECK_ARG(shares == plan.shares, "tl_gemm_rows64: %d shares do not fit this shape", shares);
     TL_CHECK_ARG(shares == 1 || partial, "tl_gemm_rows64: shares need a workspace");
-    TL_CHECK_ARG(!swiglu || (N % 2 == 0 && shares > 1), "tl_gemm_rows64: the SwiGLU form needs N even and split K");
+    TL_CHECK_ARG(!swiglu || (N % 2 == 0 && (shares > 1 || N % 32 == 0)),
+                 "tl_gemm_rows64: the SwiGLU form needs N even, and N / 2 a multiple of 16 unless K is cut");
     const int n_out = swiglu ? N / 2 : N;
     TlNormArgs na = TlNormArgs();
     if (norm) na = *norm;
@@ -384,6 +417,17 @@ extern "C" int tl_gemm_rows64(const void* A, const void* Ws, const float* bias, 
     if (M == 0) return 0;
     const int K32 = tl_ceil_div(K, 32), ntiles = tl_ceil_div(N, 16);
     float* part = shares > 1 ? partial : nullptr;
+    if (swiglu && shares == 1) {
+        // complete sums in the first kernel: a wave owns a gate tile and its up tile
+        TL_CHECK_ARG(c_dtype == TL_BF16, "tl_gemm_rows64: the paired SwiGLU form writes bfloat16");
+        const int npairs = N / 32;
+        const R64Plan pp = r64_plan_pairs(M, npairs, K);
+        hipLaunchKernelGGL((gemm_rows64_kernel<bf16_t, 4, 512, true>), dim3(pp.groups_x, 1), dim3(pp.waves * 64), 0, stream,
+                           (const bf16_t*)A, (const uint4*)Ws, nullptr, (bf16_t*)C, nullptr, M, N, K, K32, lda, ldc,
+                           pp.steps, npairs, na);
+        TL_CHECK_LAUNCH("tl_gemm_rows64 pairs");
+        return 0;
+    }
     if (c_dtype == TL_F32)
         r64_launch<float>(plan, stream, (const bf16_t*)A, (const uint4*)Ws, bias, (float*)C, part, M, N, K, K32, lda, ldc, ntiles, na);
     else

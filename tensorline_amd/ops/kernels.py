@@ -409,7 +409,7 @@ def swiglu_gate_up(h: torch.Tensor | NormedRows, gate_up_weight: torch.Tensor,
         norm, _ = _norm_args(owed, None, M, 2 * I, h.device)
         _call("tl_gemm_skinny_swiglu", _ptr(h), _ptr(shuffled), _ptr(out), M, I, K, lda, I, norm, _stream())
         return out
-    if _rows64_ok(h, shuffled, M, K, lda) and library().tl_gemm_rows64_shares(M, 2 * I, K) > 1:
+    if _rows64_ok(h, shuffled, M, K, lda) and (I % 16 == 0 or library().tl_gemm_rows64_shares(M, 2 * I, K) > 1):
         out = torch.empty(M, I, dtype=h.dtype, device=h.device)
         norm, _ = _norm_args(owed, None, M, 2 * I, h.device)
         return _rows64(h, shuffled, None, out, M, 2 * I, K, lda, I, swiglu=True, norm=norm)
