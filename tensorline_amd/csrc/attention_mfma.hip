@@ -118,12 +118,18 @@ __device__ __forceinline__ void am_block(const uint4* kf0, const uint4* kf1, con
     }
 }
 
+// index of the page that holds key k: a shift for pages of a power of two of tokens
+__device__ __forceinline__ int am_page_index(int k, int bs, int bs_shift) {
+    return bs_shift >= 0 ? k >> bs_shift : k / bs;
+}
+
 template <int DC, int NT>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, float* __restrict__ ws_o,
-    float* __restrict__ ws_ml, int nq, int nkv, int bs, int window, float scale, int nsplit, int split_blocks) {
+    float* __restrict__ ws_ml, int nq, int nkv, int bs, int bs_shift, int window, float scale, int nsplit,
+    int split_blocks) {
     constexpr int D = DC * 32;
     constexpr int DB = D / 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -188,6 +194,14 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
         for (int db = 0; db < DB; ++db) acc[j][db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
+    // The page ids of the wave's keys, one per lane, when they are at most 64 (a split of a decode
+    // step always is): a block's addresses then come from a lane exchange instead of a load from
+    // memory that the loads of keys and values would have to wait for.
+    const int page_lo = am_page_index(bb << 5, bs, bs_shift);
+    const int last_key = ((be << 5) - 1 < khi) ? (be << 5) - 1 : khi;
+    const int npages = am_page_index(last_key, bs, bs_shift) - page_lo + 1;
+    const bool pages_in_lanes = npages <= 64;
+    const int my_page = pages_in_lanes ? table[page_lo + (lane < npages ? lane : npages - 1)] : 0;
     const int krow_in_block0 = 8 * (c >> 2) + (c & 3);         // key of row c in tile 0; tile 1: + 4
     // One block ahead: while block b is multiplied, the fragments of block b + 1 are in flight
     // (past the last block the same block is requested again and not used).
@@ -200,15 +214,20 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
         int k0_ = kb_ + krow_in_block0, k1_ = k0_ + 4;                                                       \
         if (k0_ > khi) k0_ = khi;                                                                            \
         if (k1_ > khi) k1_ = khi;                                                                            \
-        const bf16_t* kp0_ = kc + ((size_t)(table[k0_ / bs] * bs + k0_ % bs) * nkv + kvh) * D + g * 8;       \
-        const bf16_t* kp1_ = kc + ((size_t)(table[k1_ / bs] * bs + k1_ % bs) * nkv + kvh) * D + g * 8;       \
+        const int i0_ = am_page_index(k0_, bs, bs_shift), i1_ = am_page_index(k1_, bs, bs_shift);            \
+        const int p0_ = pages_in_lanes ? __shfl(my_page, i0_ - page_lo, TL_WAVE) : table[i0_];               \
+        const int p1_ = pages_in_lanes ? __shfl(my_page, i1_ - page_lo, TL_WAVE) : table[i1_];               \
+        const bf16_t* kp0_ = kc + ((size_t)(p0_ * bs + k0_ - i0_ * bs) * nkv + kvh) * D + g * 8;             \
+        const bf16_t* kp1_ = kc + ((size_t)(p1_ * bs + k1_ - i1_ * bs) * nkv + kvh) * D + g * 8;             \
         _Pragma("unroll") for (int dc = 0; dc < DC; ++dc) {                                                  \
             K0[dc] = *reinterpret_cast<const uint4*>(kp0_ + dc * 32);                                        \
             K1[dc] = *reinterpret_cast<const uint4*>(kp1_ + dc * 32);                                        \
         }                                                                                                    \
         int vk_ = kb_ + 8 * g;                                                                               \
         if (vk_ > khi) vk_ = khi & ~7;                                                                       \
-        const bf16_t* vp_ = vc + (((size_t)table[vk_ / bs] * nkv + kvh) * D + c) * bs + vk_ % bs;            \
+        const int iv_ = am_page_index(vk_, bs, bs_shift);                                                    \
+        const int pv_ = pages_in_lanes ? __shfl(my_page, iv_ - page_lo, TL_WAVE) : table[iv_];               \
+        const bf16_t* vp_ = vc + (((size_t)pv_ * nkv + kvh) * D + c) * bs + vk_ - iv_ * bs;                  \
         _Pragma("unroll") for (int db = 0; db < DB; ++db)                                                    \
             V[db] = *reinterpret_cast<const uint4*>(vp_ + (size_t)db * 16 * bs);                             \
     }
@@ -580,12 +599,17 @@ static void launch_attn(int NT, dim3 grid, hipStream_t stream, const bf16_t* q, 
                         const bf16_t* vc, const int32_t* tables, int NB, const int32_t* q_start,
                         const int32_t* ctx_start, bf16_t* out, int out_stride, float* ws_o, float* ws_ml, int nq, int nkv,
                         int bs, int window, float scale, int nsplit, int split_blocks) {
+    int bs_shift = -1;                               // pages of a power of two of tokens: a shift finds the page
+    if ((bs & (bs - 1)) == 0)
+        for (bs_shift = 0; (1 << bs_shift) < bs;) ++bs_shift;
     if (NT == 1)
         hipLaunchKernelGGL((attn_mfma_kernel<DC, 1>), grid, dim3(256), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
-                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
+                           split_blocks);
     else
         hipLaunchKernelGGL((attn_mfma_kernel<DC, 2>), grid, dim3(256), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
-                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+                           ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
+                           split_blocks);
 }
 
 // q: bfloat16 [T, >= nq*d] (row stride q_stride); k_cache [pages, page, nkv, d]; v_cache
