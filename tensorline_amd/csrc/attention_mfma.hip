@@ -552,7 +552,9 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
 #undef AT_FETCH
 #undef AT_STASH
 
-// LDS of the tile kernel for head size 32 * DC and a table of `pages` page ids
+// LDS of the tile kernel for head size 32 * DC and a table of `pages` page ids: 70 KB of tiles at
+// head size 128, so two work-groups share a CU's 160 KB up to 2,560 pages per sequence and one
+// work-group has it alone beyond that
 static size_t at_lds_bytes(int DC, int pages) {
     const int D = DC * 32;
     return (size_t)(2 * AT_KEYS * (D / 8 + 1) + 2 * D * (AT_KEYS / 8 + 1)) * sizeof(uint4) + (size_t)pages * sizeof(int);
@@ -645,7 +647,7 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     dim3 grid(S, nkv, (unsigned)((waves + 3) / 4));
     const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
     const bool pow2 = (bs & (bs - 1)) == 0;
-    if (NT == 2 && nsplit == 1 && shared && pow2 && at_lds_bytes(d / 32, NB) <= 72 * 1024) {
+    if (NT == 2 && nsplit == 1 && shared && pow2 && at_lds_bytes(d / 32, NB) <= 160 * 1024) {
         // 128 columns per work-group, keys and values shared through LDS
         int bs_shift = 0;
         while ((1 << bs_shift) < bs) ++bs_shift;

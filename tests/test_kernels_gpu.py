@@ -356,6 +356,17 @@ def test_attention_portions_and_spike(dtype, nq, nkv, d, bs):
     torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
 
 
+@pytest.mark.parametrize("bs", [8, 16, 64, 128, 24])
+def test_attention_prompt_tiles_page_sizes_and_long_tables(bs):
+    """Prompt portions on the kernel that stages 64-key tiles in LDS: pages smaller than, equal to
+    and larger than a tile, a page table of more than 512 entries (8 and 16-token pages), a far key
+    that dominates, a portion that starts and ends inside a tile, a short sequence beside it.  Pages
+    of 24 tokens (no power of two) take the independent-wave kernel instead."""
+    lens, q_lens = [9000, 131, 70], [300, 131, 3]
+    got, want = _attention_case(torch.bfloat16, 28, 4, 128, bs, lens, q_lens, spike=True, seed=bs, path="mfma")
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("path", ["generic", "mfma", "mfma-direct"])
 @pytest.mark.parametrize("heads", [(14, 2), (12, 2), (16, 2), (4, 4), (28, 4)])
 @pytest.mark.parametrize("d", [32, 64, 128])
