@@ -217,7 +217,7 @@ template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict__ pos,
                                   const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   const int32_t* __restrict__ slots, int nq, int nkv, int d, int rot, int write_kv,
-                                  int bs) {
+                                  int bs, const float* __restrict__ bias) {
     __shared__ float cs_s[256], sn_s[256];          // one sine and cosine per rotated pair of the token
     const int t = blockIdx.x;
     const int half = rot / 2;
@@ -232,7 +232,11 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
         const int h = idx / half, i = idx - h * half;
         const float sn = sn_s[i], cs = cs_s[i];
         T* hp = row + (size_t)h * d;
-        const float a = tl_to_float(hp[i]), b = tl_to_float(hp[i + half]);
+        float a = tl_to_float(hp[i]), b = tl_to_float(hp[i + half]);
+        if (bias) {
+            a += bias[h * d + i];
+            b += bias[h * d + i + half];
+        }
         const T o1 = tl_from_float<T>(a * cs - b * sn);
         const T o2 = tl_from_float<T>(b * cs + a * sn);
         if (h < nq) {
@@ -244,23 +248,32 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
             kp[i + half] = o2;
         }
     }
-    if (slot < 0) return;
-    // key dims beyond the rotated part pass through
+    // dims beyond the rotated part pass through: query dims only change when a bias is owed
     const int tail = d - rot;
+    if (bias) {
+        for (int idx = threadIdx.x; idx < nq * tail; idx += blockDim.x) {
+            const int h = idx / tail, i = rot + (idx - h * tail);
+            row[(size_t)h * d + i] = tl_from_float<T>(tl_to_float(row[(size_t)h * d + i]) + bias[h * d + i]);
+        }
+    }
+    if (slot < 0) return;
     for (int idx = threadIdx.x; idx < nkv * tail; idx += blockDim.x) {
         const int h = idx / tail, i = rot + (idx - h * tail);
-        k_cache[((size_t)slot * nkv + h) * d + i] = row[(size_t)(nq + h) * d + i];
+        const T v = row[(size_t)(nq + h) * d + i];
+        k_cache[((size_t)slot * nkv + h) * d + i] = bias ? tl_from_float<T>(tl_to_float(v) + bias[(nq + h) * d + i]) : v;
     }
     // values
     const T* vrow = row + (size_t)(nq + nkv) * d;
+    const float* vbias = bias ? bias + (size_t)(nq + nkv) * d : nullptr;
     const int page = slot / bs, off = slot - page * bs;
     T* vdst = v_cache + (size_t)page * nkv * d * bs + off;
-    for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x) vdst[(size_t)idx * bs] = vrow[idx];
+    for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x)
+        vdst[(size_t)idx * bs] = vbias ? tl_from_float<T>(tl_to_float(vrow[idx]) + vbias[idx]) : vrow[idx];
 }
 
 extern "C" int tl_rope_store(void* qkv, int dtype, const int32_t* pos, const float* inv_freq, void* k_cache,
                              void* v_cache, const int32_t* slots, int T, int nq, int nkv, int d, int rot,
-                             int write_kv, int bs, hipStream_t stream) {
+                             int write_kv, int bs, const float* bias, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && nq > 0 && nkv >= 0 && d > 0, "tl_rope_store: bad sizes T=%d nq=%d nkv=%d d=%d", T, nq, nkv, d);
     TL_CHECK_ARG(rot >= 0 && rot <= d && rot % 2 == 0, "tl_rope_store: rotary width %d must be even and <= head size %d", rot, d);
     TL_CHECK_ARG(rot <= 512, "tl_rope_store: rotary width %d is above the supported 512", rot);
@@ -269,10 +282,10 @@ extern "C" int tl_rope_store(void* qkv, int dtype, const int32_t* pos, const flo
     dim3 grid(T), block(256);
     if (dtype == TL_F32)
         hipLaunchKernelGGL(rope_store_kernel<float>, grid, block, 0, stream, (float*)qkv, pos, inv_freq,
-                           (float*)k_cache, (float*)v_cache, slots, nq, nkv, d, rot, write_kv, bs);
+                           (float*)k_cache, (float*)v_cache, slots, nq, nkv, d, rot, write_kv, bs, bias);
     else if (dtype == TL_BF16)
         hipLaunchKernelGGL(rope_store_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, pos, inv_freq,
-                           (bf16_t*)k_cache, (bf16_t*)v_cache, slots, nq, nkv, d, rot, write_kv, bs);
+                           (bf16_t*)k_cache, (bf16_t*)v_cache, slots, nq, nkv, d, rot, write_kv, bs, bias);
     else
         return tl_fail("tl_rope_store: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("tl_rope_store");

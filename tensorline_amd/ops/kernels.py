@@ -474,10 +474,14 @@ def qkv_rope_store(h: torch.Tensor | NormedRows, shuffled: torch.Tensor, bias: t
 
 def rope_store(qkv: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor | None, num_heads: int,
                num_kv_heads: int, head_dim: int, k_cache: torch.Tensor | None, v_cache: torch.Tensor | None,
-               slots: torch.Tensor | None) -> None:
+               slots: torch.Tensor | None, bias: torch.Tensor | None = None) -> None:
     """Rotate the query and key heads of the fused projection ``qkv`` [T, (nq + 2 nkv) d]; queries
-    in place, rotated keys and the values into the paged cache at ``slots`` (negative: skip)."""
-    _on_gpu(qkv, pos, inv_freq, k_cache, v_cache, slots)
+    in place, rotated keys and the values into the paged cache at ``slots`` (negative: skip).
+    ``bias`` (float32, one per column of ``qkv``) is a projection bias still owed: added first."""
+    _on_gpu(qkv, pos, inv_freq, k_cache, v_cache, slots, bias)
+    if bias is not None:
+        _check(bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == qkv.shape[1],
+               "rope_store: the bias must be float32 with one entry per column")
     T = qkv.shape[0]
     width = (num_heads + 2 * num_kv_heads) * head_dim
     _check(qkv.dim() == 2 and qkv.is_contiguous() and qkv.shape[1] == width,
@@ -495,7 +499,7 @@ def rope_store(qkv: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor | No
         _i32(slots, "slots", T)
     _call("tl_rope_store", _ptr(qkv), _code(qkv, "rope_store"), _ptr(pos), _ptr(inv_freq), _ptr(k_cache), _ptr(v_cache),
           _ptr(slots), T, num_heads, num_kv_heads, head_dim, rot, 1 if write else 0,
-          k_cache.shape[1] if write else 0, _stream())
+          k_cache.shape[1] if write else 0, _ptr(bias), _stream())
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, tables: torch.Tensor,

@@ -84,10 +84,16 @@ class PagedAttention(Part):
         if fused is not None and write:
             qkv = fused(h, self.qkv, ctx.pos, self.num_heads, nkv_local, self.head_dim, cache.k, cache.v, cache.slots)
         if qkv is None:
-            qkv = self.qkv(h)
-            self.position.apply_and_store(qkv, ctx.pos, self.num_heads, nkv_local, self.head_dim,
-                                          cache.k if write else None, cache.v if write else None,
-                                          cache.slots if write else None)
+            if self.qkv.bias is not None and getattr(self.position, "adds_bias", False):
+                qkv = self.qkv(h, with_bias=False)           # the bias rides on the position encoding's pass
+                self.position.apply_and_store(qkv, ctx.pos, self.num_heads, nkv_local, self.head_dim,
+                                              cache.k if write else None, cache.v if write else None,
+                                              cache.slots if write else None, bias=self.qkv.bias)
+            else:
+                qkv = self.qkv(h)
+                self.position.apply_and_store(qkv, ctx.pos, self.num_heads, nkv_local, self.head_dim,
+                                              cache.k if write else None, cache.v if write else None,
+                                              cache.slots if write else None)
         o = kernels.paged_attention(qkv, cache.k, cache.v, cache.tables, ctx.seq_of_token, ctx.pos,
                                     self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
                                     window=self.window, q_start=ctx.q_start, ctx_start=ctx.ctx_start,

@@ -77,8 +77,9 @@ class Linear:
     def tensors_kept(self) -> list[torch.Tensor]:
         return [t for t in (self.weight, self.bias, self.shuffled) if t is not None]
 
-    def __call__(self, x, out_dtype: torch.dtype | None = None, sink=None):
-        return kernels.linear(x, self.weight, self.bias, out_dtype=out_dtype, shuffled=self.shuffled, sink=sink)
+    def __call__(self, x, out_dtype: torch.dtype | None = None, sink=None, with_bias: bool = True):
+        return kernels.linear(x, self.weight, self.bias if with_bias else None, out_dtype=out_dtype,
+                              shuffled=self.shuffled, sink=sink)
 
 
 def fuse_linears(name: str, parts: list[Linear]) -> Linear:

@@ -4,7 +4,9 @@ cache (fused, because the rotated key is what the cache holds; reference: paged.
 
 Interface: ``apply_and_store(qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
 slots)`` rotates the query heads of the fused projection in place and stores keys and values at
-``slots`` (``k_cache`` None: nothing is stored).  A position encoding may also offer
+``slots`` (``k_cache`` None: nothing is stored).  One that sets ``adds_bias`` also takes
+``bias=``, the projection's bias still to be added (the mixer then leaves it out of the product:
+one pass over the activations less).  A position encoding may also offer
 ``project_rotate_store(h, qkv_linear, ...)``, which does the projection as well and returns the
 queries, or None to decline; the attention mixer tries it first.
 """
@@ -33,8 +35,10 @@ class RotaryEmbedding:
         inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -idx / self.rotary_dim)
         self.inv_freq = inv.to(torch.float32).to(device)
 
-    def apply_and_store(self, qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots) -> None:
-        kernels.rope_store(qkv, pos, self.inv_freq, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots)
+    adds_bias = True     # apply_and_store takes the projection's bias and adds it on the way
+
+    def apply_and_store(self, qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots, bias=None) -> None:
+        kernels.rope_store(qkv, pos, self.inv_freq, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots, bias)
 
     def project_rotate_store(self, h, qkv_linear, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots):
         """Optional shortcut for few-row steps: projection, rotation and cache write in one kernel.
@@ -52,6 +56,8 @@ class NoPosition:
     def __init__(self, head_dim: int, device):
         self.head_dim = int(head_dim)
 
-    def apply_and_store(self, qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots) -> None:
-        if k_cache is not None:
-            kernels.rope_store(qkv, pos, None, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots)
+    adds_bias = True
+
+    def apply_and_store(self, qkv, pos, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots, bias=None) -> None:
+        if k_cache is not None or bias is not None:
+            kernels.rope_store(qkv, pos, None, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots, bias)

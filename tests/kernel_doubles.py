@@ -49,9 +49,11 @@ def linear(a, weight, bias=None, out_dtype=None, out=None, shuffled=None, sink=N
     return y.to(out_dtype or a.dtype)
 
 
-def rope_store(qkv, pos, inv_freq, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots):
+def rope_store(qkv, pos, inv_freq, num_heads, num_kv_heads, head_dim, k_cache, v_cache, slots, bias=None):
     T = qkv.shape[0]
     d = head_dim
+    if bias is not None:
+        qkv.copy_((qkv.to(torch.float32) + bias).to(qkv.dtype))
     heads = qkv.view(T, num_heads + 2 * num_kv_heads, d)
     rot_heads = heads[:, :num_heads + num_kv_heads].to(torch.float32)
     if inv_freq is not None and inv_freq.numel():

@@ -157,6 +157,19 @@ def test_rope_store(dtype, nq, nkv, d, rot):
     keep = qkv0.clone()
     K().rope_store(qkv0, torch.zeros(3, dtype=torch.int32, device=DEV), inv_freq, nq, nkv, d, None, None, None)
     torch.testing.assert_close(qkv0, keep, atol=0, rtol=0)
+    # an owed bias: the same as adding it beforehand (in float32: to the bit)
+    bias = torch.randn((nq + 2 * nkv) * d, device=DEV)
+    outs = []
+    for owed in (True, False):
+        x = qkv.clone() if owed else (qkv.float() + bias).to(dtype)      # qkv holds rotated queries by now: any input will do
+        kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+        K().rope_store(x, pos, inv_freq, nq, nkv, d, kc2, vc2, slots, bias if owed else None)
+        outs.append((x[:, :nq * d], kc2, vc2))
+    for a, b in zip(*outs):
+        if dtype == torch.float32:
+            torch.testing.assert_close(a, b, atol=0, rtol=0)
+        else:
+            torch.testing.assert_close(a.float(), b.float(), atol=3e-2, rtol=3e-2)
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64])
