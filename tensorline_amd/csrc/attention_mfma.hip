@@ -562,7 +562,7 @@ static size_t at_lds_bytes(int DC, int pages) {
 
 // Merge the splits of one (token, head): M = max m_s, out = sum acc_s e^(m_s - M) / sum l_s e^(m_s - M),
 // over the splits that hold keys of the token, in ascending order.
-#define AM_MAX_SPLITS 256
+#define AM_MAX_SPLITS 1024
 __global__ void attn_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                   const int32_t* __restrict__ pos, bf16_t* __restrict__ out, int out_stride, int nq,
                                   int D, int nsplit, int split_blocks, int window) {

@@ -284,6 +284,7 @@ def linear(a: torch.Tensor | NormedRows, weight: torch.Tensor, bias: torch.Tenso
     return _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled)
 
 
+MAX_KEY_SPLITS = 1024    # key splits the attention merge kernel takes
 SKINNY_MAX_ROWS = 16     # rows the few-row kernel serves (one 16-row MFMA tile)
 ROWS64_MAX_ROWS = 64     # rows the 17..64-row kernel serves; above that the library
 
@@ -559,6 +560,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         nsplit, split_blocks = 1, 1
         if split_len:
             _check(split_len % 32 == 0, "paged_attention: a split is a multiple of 32 keys")
+            while -(-plan.max_context // split_len) > MAX_KEY_SPLITS:    # very long contexts: longer splits
+                split_len *= 2
             split_blocks = split_len // 32
             nsplit = max(1, -(-plan.max_context // split_len))
         ws_o = ws_ml = None

@@ -369,6 +369,14 @@ def test_attention_portions_and_spike(dtype, nq, nkv, d, bs):
     torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
 
 
+@pytest.mark.parametrize("lens,split", [([33000], None), ([70001, 9], None), ([70001], 32)])
+def test_attention_decode_long_contexts(lens, split):
+    """Decoded tokens over tens of thousands of keys: hundreds of key splits, and beyond the most
+    splits the merge takes the splits grow; a far key dominates."""
+    got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, lens, None, spike=True, seed=5, path="mfma", split_keys=split)
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("bs", [8, 16, 64, 128, 24])
 def test_attention_prompt_tiles_page_sizes_and_long_tables(bs):
     """Prompt portions on the kernel that stages 64-key tiles in LDS: pages smaller than, equal to
