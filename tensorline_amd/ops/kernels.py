@@ -609,9 +609,12 @@ def argmax(logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tenso
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, uniform: torch.Tensor,
-           out: torch.Tensor | None = None) -> torch.Tensor:
+           out: torch.Tensor | None = None, any_top_p: bool | None = None, any_greedy: bool = True) -> torch.Tensor:
     """One token per row of float32 logits [R, V]: greedy where temperature <= 0, else a draw from
-    softmax(logits / temperature) cut by top-p, using the uniform number given for the row."""
+    softmax(logits / temperature) cut by top-p, using the uniform number given for the row.
+    ``any_top_p``: whether some row has top_p < 1, if the caller knows (saves three kernels when
+    none has, and a look at the device when not given); ``any_greedy`` False promises that no row
+    is greedy (saves the arg-max)."""
     _on_gpu(logits, temperature, top_p, uniform, out)
     _check(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be float32 [R, V]")
     R, V = logits.shape
@@ -620,6 +623,11 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
     if out is None:
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
     _i32(out, "sample output", R)
+    if any_top_p is None:
+        any_top_p = bool((top_p < 1).any().item())
+    chunks = library().tl_sample_chunks(V)
+    pmax = torch.empty(R * chunks, dtype=torch.float32, device=logits.device)
+    ws = torch.zeros(R * (3080 + 3 * chunks), dtype=torch.int64, device=logits.device)
     _call("tl_sample", _ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature), _ptr(top_p),
-          _ptr(uniform), _ptr(out), _stream())
+          _ptr(uniform), _ptr(out), _ptr(pmax), _ptr(ws), 1 if any_greedy else 0, 1 if any_top_p else 0, _stream())
     return out

@@ -41,4 +41,6 @@ class Sampler:
             return kernels.argmax(logits).tolist()
         u = [uniform_for(s, i) for s, i in zip(seeds, indices)]
         params = torch.tensor([temperatures, top_ps, u], dtype=torch.float32).to(self.device)
-        return kernels.sample(logits, params[0], params[1], params[2]).tolist()
+        return kernels.sample(logits, params[0], params[1], params[2],
+                              any_top_p=any(p < 1.0 for p in top_ps),
+                              any_greedy=any(t <= 0 for t in temperatures)).tolist()

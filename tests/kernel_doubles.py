@@ -108,7 +108,7 @@ def argmax(logits, out=None):
     return logits.argmax(-1).to(torch.int32)
 
 
-def sample(logits, temperature, top_p, uniform, out=None):
+def sample(logits, temperature, top_p, uniform, out=None, any_top_p=None, any_greedy=True):
     res = torch.empty(logits.shape[0], dtype=torch.int32)
     for r in range(logits.shape[0]):
         t = float(temperature[r])

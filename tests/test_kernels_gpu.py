@@ -491,6 +491,50 @@ def test_sample_keep_rule_and_draws():
     assert again.tolist() == got[10:20]
 
 
+def test_sample_wide_rows_ties_and_masked_logits():
+    """Rows of several chunks: agreement with the plain rule, a row of equal logits (the kept set is
+    a number of ties, lowest indices first), a row with all but two logits at -inf, a dominant token."""
+    torch.manual_seed(4)
+    V = 10007
+    R = 12
+    lg = torch.randn(R, V, device=DEV) * 4
+    temp = torch.rand(R, device=DEV) * 1.2 + 0.2
+    tp = torch.rand(R, device=DEV) * 0.95 + 0.04
+    tp[::4] = 1.0
+    u = torch.rand(R, device=DEV)
+    got = K().sample(lg, temp, tp, u).tolist()
+    miss = 0
+    for r in range(R):
+        want = plain.sample_with_uniform(lg[r].cpu(), float(temp[r]), float(tp[r]), float(u[r]))
+        if got[r] != want:
+            probs = torch.softmax(lg[r].double().cpu() / float(temp[r]), -1)
+            if tp[r] < 1:
+                assert plain.top_p_keep(probs, float(tp[r]))[got[r]], "drew a token outside the kept set"
+            miss += 1
+    assert miss <= 1
+    # equal logits: top_p 0.3 keeps tokens while k / V < 0.3, that is the first 3003; u picks evenly among them
+    us = torch.tensor([0.0, 0.25, 0.5, 0.999999], device=DEV)
+    n = us.numel()
+    flat = torch.zeros(n, V, device=DEV)
+    got = K().sample(flat, torch.ones(n, device=DEV), torch.full((n,), 0.3, device=DEV), us).tolist()
+    assert got == [int(float(x) * 3003) for x in us.tolist()]
+    got = K().sample(flat, torch.ones(n, device=DEV), torch.ones(n, device=DEV), us).tolist()
+    assert got == [int(float(x) * V) for x in us.tolist()]
+    # two live tokens far apart, the rest -inf: p = (0.25, 0.75)
+    two = torch.full((3, V), float("-inf"), device=DEV)
+    two[:, 5000] = math.log(0.25)
+    two[:, 9999] = math.log(0.75)
+    one = torch.ones(3, device=DEV)
+    assert K().sample(two, one, one, torch.tensor([0.1, 0.3, 0.9], device=DEV)).tolist() == [5000, 9999, 9999]
+    assert K().sample(two, one, one * 0.7, torch.tensor([0.1, 0.3, 0.9], device=DEV)).tolist() == [9999] * 3
+    # the vocabulary of the 7B shape: a dominant token wins whatever u is
+    big = torch.randn(2, 152064, device=DEV)
+    big[0, 151000] = 60.0
+    big[1, 3] = 60.0
+    assert K().sample(big, torch.ones(2, device=DEV), torch.tensor([0.9, 1.0], device=DEV),
+                      torch.tensor([0.9999, 0.5], device=DEV)).tolist() == [151000, 3]
+
+
 def test_sample_frequencies():
     torch.manual_seed(2)
     V, R = 50, 20000
