@@ -185,6 +185,11 @@ class CacheManager:
                                        arrays=[None] * len(self.groups), serial=self._serial)
         return slot
 
+    @property
+    def has_windows(self) -> bool:
+        """Whether some group gives pages back while a request lives (a windowed group)."""
+        return self._windowed
+
     def admission(self, rid) -> int:
         """A number that differs between two admissions of a request id (its pages were given back
         in between): whoever keeps a copy of a table can tell that it is stale."""

@@ -144,6 +144,7 @@ extern "C" int tl_argmax(const float* logits, int ld, int R, int V, int32_t* out
 #define SP_STATE (3 * SP_BUCKETS)            // per row: three mass histograms, then 8 state words
 #define SP_ROW_WORDS (SP_STATE + 8)          // state: P, bucket and mass above of levels 1 and 2, w_t's bits, mass above w_t
 typedef unsigned long long u64;
+static_assert(SP_BUCKETS == 4 * SP_THREADS, "sp_find gives four buckets to a thread");
 
 __device__ __forceinline__ u64 sp_fix(float w) { return (w > 0.f) ? (u64)(w * 1099511627776.0f) : 0ull; }
 

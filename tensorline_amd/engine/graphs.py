@@ -131,7 +131,7 @@ class GraphRunner(ModelRunner):
         position, cache row, and a page id where a request entered a new page) instead of being
         packed again.  False: not that case, nothing was touched."""
         cache = self.cache
-        if cap.rids is None or len(cap.rids) != len(entries) or cache._windowed:
+        if cap.rids is None or len(cap.rids) != len(entries) or cache.has_windows:
             return False
         for rid, adm, e in zip(cap.rids, cap.admissions, entries):
             if e.rid != rid or cache.admission(rid) != adm:  # another request, or the same one admitted again
