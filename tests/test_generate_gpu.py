@@ -43,6 +43,22 @@ def test_greedy_generation_matches_plain(folder_b, greedy_want, opts):
         assert c["preemptions"] > 0
 
 
+@pytest.mark.parametrize("block_size", [16, 32, 64, 128])
+def test_greedy_generation_with_other_page_sizes(folder_b, greedy_want, block_size):
+    """Pages larger than the kernels' key blocks and tiles: 32-bit tokens equal the plain ones, and
+    bfloat16 agrees with 32-bit on most tokens."""
+    from tensorline_amd import LLM, SamplingParams
+    d, w, cfg = folder_b
+    prompts, want = greedy_want
+    sp = SamplingParams(max_tokens=24, stop_token_ids=NO_STOP)
+    llm = LLM(d, dtype="float32", device=DEV, num_blocks=2048 // block_size, block_size=block_size, max_batched_tokens=48)
+    assert [o.token_ids for o in llm.generate(prompts, sp)] == want
+    llm = LLM(d, dtype="bfloat16", device=DEV, num_blocks=2048 // block_size, block_size=block_size, max_batched_tokens=48)
+    got = [o.token_ids for o in llm.generate(prompts, sp)]
+    same = sum(a == b for g, x in zip(got, want) for a, b in zip(g, x))
+    assert same >= 0.6 * sum(len(x) for x in want)
+
+
 def test_bfloat16_generation_same_with_and_without_graphs(folder_b, greedy_want):
     from tensorline_amd import LLM, SamplingParams
     d, w, cfg = folder_b
