@@ -44,6 +44,7 @@ __device__ __forceinline__ uint32_t am_pack2(float a, float b) {
 }
 
 #define AM_LOG2E 1.4426950408889634f
+#define AM_LAZY 8.0f                 // how far a block's maximum may exceed the running one before it moves
 #define AM_NO_COLUMN 0x7fffffff      // position of a lane without a column: never masks, never written
 
 // One block of 32 keys for the NT column tiles of a wave: scores, online softmax, P*V.
@@ -324,9 +325,13 @@ __device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, c
         float bmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
         bmax = fmaxf(bmax, __shfl_xor(bmax, 16, TL_WAVE));
         bmax = fmaxf(bmax, __shfl_xor(bmax, 32, TL_WAVE));
-        const float m_new = fmaxf(m_run[j], bmax);
+        // The running maximum follows the true one lazily: it moves only when the block's maximum
+        // exceeds it by more than AM_LAZY (in the base-2 domain), so probabilities stay below
+        // 2^AM_LAZY and the accumulator is rescaled in few blocks instead of most.  Sums and
+        // accumulators stay relative to the same running maximum, so the result is the same.
+        const bool moved = bmax > m_run[j] + AM_LAZY || (m_run[j] == -INFINITY && bmax > -INFINITY);
+        const float m_new = moved ? bmax : m_run[j];
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const bool moved = m_new > m_run[j];
         float pr[8], psum = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -361,30 +366,34 @@ __device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, c
     }
 }
 
-// The kernel for steps with prompt portions.  A work-group of four waves owns 128 consecutive
-// columns of one (sequence, key/value head), 32 per wave, and walks the keys together in tiles of
-// 64.  A tile is brought into LDS once, with contiguous loads (whole key rows of K, runs of keys of
-// one dim of V^T), and every wave takes its MFMA fragments from there: keys and values are read
-// from the cache once per 128 columns, and a wave holds no copy of them in registers, so two
-// work-groups fit on a CU and one computes while the other waits.  Two LDS buffers: the loads of
-// tile t + 1 are in flight (in registers) while tile t is multiplied, and go to the other buffer
-// before the one barrier of the iteration.  The sequence's page ids are copied to LDS first, so a
-// tile's addresses depend on no load from memory.  Pages must hold a power of two of tokens (at
-// least 8; 2^bs_shift): an 8-key run of V^T then lies in one page and a page id is a shift away.
-// No key split: a step with prompt portions has columns enough.
+// The kernel for steps with prompt portions.  A work-group owns 128 consecutive columns of one
+// (sequence, key/value head), 16 * NT per wave, and walks the keys together in tiles of 64.  A
+// tile is brought into LDS once, with contiguous loads (whole key rows of K, runs of keys of one
+// dim of V^T), and every wave takes its MFMA fragments from there: keys and values are read from
+// the cache once per 128 columns, and a wave holds no copy of them in registers, so two
+// work-groups (sixteen waves) fit on a CU and some compute while others wait.  Two LDS buffers:
+// the loads of tile t + 1 are in flight (in registers) while tile t is multiplied, and go to the
+// other buffer before the one barrier of the iteration.  The sequence's page ids are copied to
+// LDS first, so a tile's addresses depend on no load from memory.  Pages must hold a power of two
+// of tokens (at least 8; 2^bs_shift): an 8-key run of V^T then lies in one page and a page id is
+// a shift away.  No key split: a step with prompt portions has columns enough.  (Measured on a
+// 2,048-token prompt at 28/4 heads of 128: 86 us with one column tile on each of eight waves, 98 us
+// with two on each of four; the time is that of the last group, which walks all the keys.)
 #define AT_KEYS 64
+#define AT_NT 1                      // column tiles per wave; 8 / AT_NT waves in a work-group
 // LDS row of key k of a tile (see am_block_lds)
 __device__ __forceinline__ int at_lds_row(int k) {
     return (k & 32) + ((k & 4) << 2) + ((k & 24) >> 1) + (k & 3);
 }
 
-template <int DC>
-__global__ __launch_bounds__(256, 2) void attn_tile_kernel(
+template <int DC, int NT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int nq, int nkv, int bs,
     int bs_shift, int window, float scale) {
-    constexpr int NT = 2;
+    constexpr int THREADS = WAVES * 64;
+    constexpr int WCOLS = NT * 16;                       // columns of a wave; WAVES * WCOLS = 128 per work-group
     constexpr int D = DC * 32;
     constexpr int DB = D / 16;
     constexpr int KP = D / 8 + 1;             // uint4 per key row in LDS (one of padding)
@@ -402,10 +411,32 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
     const int n = q_start[s + 1] - r0;
     const int start = ctx_start[s];
     const int ncols = n * G;
+    // Loader.  A K tile is 64 keys x D/8 units of 16 bytes, a V^T tile D dims x 8 units (8 keys
+    // each): LU units of each per thread (threads past the last unit repeat it and store nothing).
+    // K: consecutive threads take consecutive units of a key row.  V^T: consecutive threads take
+    // the units of one dim inside a page, then the next dim, which is how a page lies in memory
+    // ([dim][token]); `opp` units of a dim are in one page.
+    const int opp_shift = (bs_shift < 6) ? bs_shift - 3 : 3;    // log2(min(bs, 64) / 8)
+    constexpr int UPK = D / 8;                               // units per key row
+    constexpr int UNITS = AT_KEYS * UPK;                     // units of a K tile, and of a V^T tile
+    constexpr int LU = (UNITS + THREADS - 1) / THREADS;
+    int k_at[LU], v_at[LU];                                  // key | unit << 16;  dim | first key of the unit << 16
+    bool u_mine[LU];
+#pragma unroll
+    for (int i = 0; i < LU; ++i) {
+        int u = tid + THREADS * i;
+        u_mine[i] = u < UNITS;
+        if (!u_mine[i]) u = UNITS - 1;
+        k_at[i] = (u / UPK) | ((u % UPK) << 16);
+        const int o = u & ((1 << opp_shift) - 1);
+        const int rest = u >> opp_shift;
+        v_at[i] = (rest % D) | (((((rest / D) << opp_shift) + o) * 8) << 16);
+    }
+    uint4 kreg[LU], vreg[LU];
     // the groups with the most keys (the last columns) start first
     const int wg_col0 = (int)(gridDim.z - 1 - blockIdx.z) * 128;
     if (wg_col0 >= ncols) return;             // the whole work-group leaves: no barrier is missed
-    const int col0 = wg_col0 + wave * 32;
+    const int col0 = wg_col0 + wave * WCOLS;
     const bool wave_active = col0 < ncols;
 
     // key range of the work-group and of this wave
@@ -419,7 +450,7 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
     const int t_lo = klo / AT_KEYS, t_hi = khi / AT_KEYS;
     int wk_lo = 1, wk_hi = 0;                 // empty for a wave without columns
     if (wave_active) {
-        const int w_last = ((col0 + 32 < ncols) ? col0 + 32 : ncols) - 1;
+        const int w_last = ((col0 + WCOLS < ncols) ? col0 + WCOLS : ncols) - 1;
         wk_hi = start + w_last / G;
         wk_lo = 0;
         if (window > 0) {
@@ -431,7 +462,7 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
     {
         const int32_t* table = tables + (size_t)s * NB;
         const int npages = (khi >> bs_shift) + 1;
-        for (int i = tid; i < npages; i += 256) tab[i] = table[i];
+        for (int i = tid; i < npages; i += THREADS) tab[i] = table[i];
     }
 
     uint4 qf[NT][DC];
@@ -464,36 +495,20 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
         for (int db = 0; db < DB; ++db) acc[j][db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // Loader.  A K tile is 64 keys x D/8 units of 16 bytes, a V^T tile D dims x 8 units (8 keys
-    // each): DC units of each per thread.  K: consecutive threads take consecutive units of a key
-    // row.  V^T: consecutive threads take the units of one dim inside a page, then the next dim,
-    // which is how a page lies in memory ([dim][token]); `opp` units of a dim are in one page.
-    const int opp_shift = (bs_shift < 6) ? bs_shift - 3 : 3;    // log2(min(bs, 64) / 8)
-    constexpr int UPK = D / 8;                               // units per key row
-    const int k_key0 = tid / UPK, k_unit = tid % UPK;        // unit i of the thread: key k_key0 + i * 256 / UPK
-    int v_at[DC];                                            // dim | first key of the unit within the tile << 16
-#pragma unroll
-    for (int i = 0; i < DC; ++i) {
-        const int u = tid + 256 * i;
-        const int o = u & ((1 << opp_shift) - 1);
-        const int rest = u >> opp_shift;
-        v_at[i] = (rest % D) | (((((rest / D) << opp_shift) + o) * 8) << 16);
-    }
-    uint4 kreg[DC], vreg[DC];
 #define AT_PAGE(KEY, PG, OFF)                                                                                  \
     OFF = (KEY) & (bs - 1);                                                                                   \
     PG = tab[(KEY) >> bs_shift];
 #define AT_FETCH(T)                                                                                            \
     {                                                                                                         \
         const int kb_ = (T) * AT_KEYS;                                                                        \
-        _Pragma("unroll") for (int i = 0; i < DC; ++i) {                                                      \
-            int key_ = kb_ + k_key0 + i * (256 / UPK);                                                        \
+        _Pragma("unroll") for (int i = 0; i < LU; ++i) {                                                      \
+            int key_ = kb_ + (k_at[i] & 0xffff);                                                              \
             if (key_ > khi) key_ = khi; /* masked for every column; stay on owned pages */                    \
             int pg_, off_;                                                                                    \
             AT_PAGE(key_, pg_, off_)                                                                          \
-            kreg[i] = *reinterpret_cast<const uint4*>(kc + ((size_t)(pg_ * bs + off_) * nkv + kvh) * D + k_unit * 8); \
+            kreg[i] = *reinterpret_cast<const uint4*>(kc + ((size_t)(pg_ * bs + off_) * nkv + kvh) * D + (k_at[i] >> 16) * 8); \
         }                                                                                                     \
-        _Pragma("unroll") for (int i = 0; i < DC; ++i) {                                                      \
+        _Pragma("unroll") for (int i = 0; i < LU; ++i) {                                                      \
             int vk_ = kb_ + (v_at[i] >> 16);                                                                  \
             if (vk_ > khi) vk_ = khi & ~7;                                                                    \
             int pg_, off_;                                                                                    \
@@ -503,9 +518,11 @@ __global__ __launch_bounds__(256, 2) void attn_tile_kernel(
     }
 #define AT_STASH(BUF)                                                                                          \
     {                                                                                                         \
-        _Pragma("unroll") for (int i = 0; i < DC; ++i) {                                                      \
-            ks[(BUF) * AT_KEYS * KP + at_lds_row(k_key0 + i * (256 / UPK)) * KP + k_unit] = kreg[i];           \
-            vs[(BUF) * D * VP + (v_at[i] & 0xffff) * VP + (v_at[i] >> 19)] = vreg[i];                          \
+        _Pragma("unroll") for (int i = 0; i < LU; ++i) {                                                      \
+            if (u_mine[i]) {                                                                                  \
+                ks[(BUF) * AT_KEYS * KP + at_lds_row(k_at[i] & 0xffff) * KP + (k_at[i] >> 16)] = kreg[i];      \
+                vs[(BUF) * D * VP + (v_at[i] & 0xffff) * VP + (v_at[i] >> 19)] = vreg[i];                      \
+            }                                                                                                 \
         }                                                                                                     \
     }
 
@@ -651,11 +668,12 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
         // 128 columns per work-group, keys and values shared through LDS
         int bs_shift = 0;
         while ((1 << bs_shift) < bs) ++bs_shift;
-        dim3 sgrid(S, nkv, (unsigned)((max_tile_groups + 3) / 4));
+        dim3 sgrid(S, nkv, (unsigned)((max_tile_groups + 3) / 4));   // the caller counts groups of 32 columns
         const size_t lds = at_lds_bytes(d / 32, NB);
 #define TL_TILE_CASE(DCV)                                                                                             \
-    hipLaunchKernelGGL((attn_tile_kernel<DCV>), sgrid, dim3(256), lds, stream, qq, q_stride, kk, vv, tables, NB,       \
-                       q_start, ctx_start, (bf16_t*)out, out_stride, nq, nkv, bs, bs_shift, window, scale)
+    hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT>), sgrid, dim3(64 * 8 / AT_NT), lds, stream, qq,        \
+                       q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, nq, nkv, bs,        \
+                       bs_shift, window, scale)
         if (d == 32) TL_TILE_CASE(1);
         else if (d == 64) TL_TILE_CASE(2);
         else TL_TILE_CASE(4);
