@@ -390,7 +390,7 @@ template <int DC, int NT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
-    const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int nq, int nkv, int bs,
+    const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int S, int nq, int nkv, int bs,
     int bs_shift, int window, float scale) {
     constexpr int THREADS = WAVES * 64;
     constexpr int WCOLS = NT * 16;                       // columns of a wave; WAVES * WCOLS = 128 per work-group
@@ -401,14 +401,28 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
     extern __shared__ uint4 at_smem[];
     uint4* ks = at_smem;                                   // [2][AT_KEYS * KP]
     uint4* vs = at_smem + 2 * AT_KEYS * KP;                // [2][D * VP]
-    int* tab = reinterpret_cast<int*>(vs + 2 * D * VP);    // page ids of the sequence, as far as needed
+    int* tab = reinterpret_cast<int*>(vs + 2 * D * VP);    // page ids of the sequence, as far as needed (NB ints)
+    int* qst = tab + NB;                                   // q_start of the step (S + 1 ints)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
-    const int s = blockIdx.x, kvh = blockIdx.y;
+    const int kvh = blockIdx.x;                            // fastest: the heads of a group start together
     const int G = nq / nkv;
     const float scale2 = scale * AM_LOG2E;
-    const int r0 = q_start[s];
-    const int n = q_start[s + 1] - r0;
+    // Which (sequence, group of 128 columns) this work-group owns: the grid has one work-group per
+    // group that exists (a step mixes a long prompt portion with many one-token sequences, and a
+    // grid of sequences x most groups would be nearly all empty work-groups).  Within a sequence
+    // the groups with the most keys (the last columns) come first.
+    for (int i = tid; i <= S; i += THREADS) qst[i] = q_start[i];
+    __syncthreads();
+    int s = 0, flat = blockIdx.y, ngroups = 0;
+    for (; s < S; ++s) {
+        ngroups = ((qst[s + 1] - qst[s]) * G + 127) / 128;
+        if (flat < ngroups) break;
+        flat -= ngroups;
+    }
+    if (s >= S) return;                       // the whole work-group leaves: no barrier is missed
+    const int r0 = qst[s];
+    const int n = qst[s + 1] - r0;
     const int start = ctx_start[s];
     const int ncols = n * G;
     // Loader.  A K tile is 64 keys x D/8 units of 16 bytes, a V^T tile D dims x 8 units (8 keys
@@ -433,9 +447,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
         v_at[i] = (rest % D) | (((((rest / D) << opp_shift) + o) * 8) << 16);
     }
     uint4 kreg[LU], vreg[LU];
-    // the groups with the most keys (the last columns) start first
-    const int wg_col0 = (int)(gridDim.z - 1 - blockIdx.z) * 128;
-    if (wg_col0 >= ncols) return;             // the whole work-group leaves: no barrier is missed
+    const int wg_col0 = (ngroups - 1 - flat) * 128;
     const int col0 = wg_col0 + wave * WCOLS;
     const bool wave_active = col0 < ncols;
 
@@ -569,12 +581,13 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
 #undef AT_FETCH
 #undef AT_STASH
 
-// LDS of the tile kernel for head size 32 * DC and a table of `pages` page ids: 70 KB of tiles at
+// LDS of the tile kernel for head size 32 * DC, a table of `pages` page ids and S sequences: 70 KB of tiles at
 // head size 128, so two work-groups share a CU's 160 KB up to 2,560 pages per sequence and one
 // work-group has it alone beyond that
-static size_t at_lds_bytes(int DC, int pages) {
+static size_t at_lds_bytes(int DC, int pages, int S) {
     const int D = DC * 32;
-    return (size_t)(2 * AT_KEYS * (D / 8 + 1) + 2 * D * (AT_KEYS / 8 + 1)) * sizeof(uint4) + (size_t)pages * sizeof(int);
+    return (size_t)(2 * AT_KEYS * (D / 8 + 1) + 2 * D * (AT_KEYS / 8 + 1)) * sizeof(uint4) +
+           (size_t)(pages + S + 1) * sizeof(int);
 }
 
 // Merge the splits of one (token, head): M = max m_s, out = sum acc_s e^(m_s - M) / sum l_s e^(m_s - M),
@@ -639,11 +652,12 @@ static void launch_attn(int NT, dim3 grid, hipStream_t stream, const bf16_t* q, 
 // (the tokens' positions), ws_o holds T*nq*nsplit*d floats and ws_ml T*nq*nsplit*2.  shared != 0
 // runs unsplit steps with prompt portions on the kernel that shares keys and values through LDS
 // (when the page size and the table length allow it); shared == 0 keeps them on independent waves.
+// total_groups128: the sum over the sequences of ceil(n_s * G / 128), that kernel's grid.
 extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int32_t* tables, int NB, const int32_t* q_start, const int32_t* ctx_start,
                                  const int32_t* pos, void* out, int out_stride, float* ws_o, float* ws_ml, int T, int S,
                                  int nq, int nkv, int d, int bs, int window, float scale, int NT, int max_tile_groups,
-                                 int nsplit, int split_blocks, int shared, hipStream_t stream) {
+                                 int nsplit, int split_blocks, int shared, int total_groups128, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && NB > 0, "tl_attention_mfma: bad sizes T=%d S=%d nq=%d nkv=%d NB=%d", T, S, nq, nkv, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_mfma: %d query heads are not a multiple of %d key/value heads", nq, nkv);
     TL_CHECK_ARG(d == 32 || d == 64 || d == 128, "tl_attention_mfma: head size %d is not one of 32, 64, 128", d);
@@ -664,15 +678,16 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     dim3 grid(S, nkv, (unsigned)((waves + 3) / 4));
     const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
     const bool pow2 = (bs & (bs - 1)) == 0;
-    if (NT == 2 && nsplit == 1 && shared && pow2 && at_lds_bytes(d / 32, NB) <= 160 * 1024) {
+    if (NT == 2 && nsplit == 1 && shared && pow2 && total_groups128 > 0 && at_lds_bytes(d / 32, NB, S) <= 160 * 1024) {
         // 128 columns per work-group, keys and values shared through LDS
         int bs_shift = 0;
         while ((1 << bs_shift) < bs) ++bs_shift;
-        dim3 sgrid(S, nkv, (unsigned)((max_tile_groups + 3) / 4));   // the caller counts groups of 32 columns
-        const size_t lds = at_lds_bytes(d / 32, NB);
+        TL_CHECK_ARG(total_groups128 <= 65535, "tl_attention_mfma: %d column groups are more than a launch takes", total_groups128);
+        dim3 sgrid(nkv, (unsigned)total_groups128, 1);
+        const size_t lds = at_lds_bytes(d / 32, NB, S);
 #define TL_TILE_CASE(DCV)                                                                                             \
     hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT>), sgrid, dim3(64 * 8 / AT_NT), lds, stream, qq,        \
-                       q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, nq, nkv, bs,        \
+                       q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, S, nq, nkv, bs,     \
                        bs_shift, window, scale)
         if (d == 32) TL_TILE_CASE(1);
         else if (d == 64) TL_TILE_CASE(2);

@@ -547,6 +547,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         groups = [-(-n * G // (16 * nt)) for n in plan.q_lens]
         pads = max(0, S - len(groups))                     # padding sequences bring one token each
         max_groups = max(groups + [1])
+        total128 = sum(-(-n * G // 128) for n in plan.q_lens) + pads
         # Splits are fixed runs of keys aligned to absolute positions, so the same keys are summed
         # together whatever the context length or the launch shape.  Pure decode steps split by the
         # batch size rounded up to a power of two (what a graph bucket pads to); steps with prompt
@@ -571,7 +572,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
               _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,
               num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,
-              0 if path == "mfma-direct" else 1, _stream())
+              0 if path == "mfma-direct" else 1, total128, _stream())
         return out
     _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
           _ptr(seq_of_token), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, num_heads,
