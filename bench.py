@@ -7,7 +7,9 @@ A step is one decode step of the whole batch through the engine loop (schedule, 
 of the model, sampling, accept).  Weights are random (generated on the GPU from a seed), prompts
 are token ids uniform over the vocabulary.  One JSON line is printed: decoded tokens per second
 at the default batch, the prefill of one 2,048-token prompt, the decode step's share of the HBM
-roofline, and decode throughput at batch 1 and 64.
+roofline, and decode throughput at batch 1 and 64.  The fractions are of the published peaks;
+``machine`` holds what this GPU reaches on a plain copy and on a large library product, and the
+``frac_of_measured_*`` fields are the same figures relative to those.
 """
 from __future__ import annotations
 
@@ -146,6 +148,34 @@ def bench_prefill(llm, tokens: int, reps: int, seed: int) -> dict:
     return {"s": best, "tok_s": tokens / best}
 
 
+def measure_machine(dtype) -> dict:
+    """What this GPU reaches on two plain jobs, beside the published peaks: a device-to-device
+    copy of 2 GiB (bytes read plus bytes written per second) and a square library product of
+    8,192 rows in the benchmark's dtype (float32: the library's true 32-bit kernels)."""
+    import torch
+    src = torch.empty(1 << 30, dtype=torch.int16, device="cuda:0").fill_(1)
+    dst = torch.empty_like(src)
+    n = 8192
+    a = torch.randn(n, n, dtype=dtype, device="cuda:0")
+    b = torch.randn(n, n, dtype=dtype, device="cuda:0")
+
+    def best_ms(fn, reps):
+        fn()
+        best = float("inf")
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            e1.synchronize()
+            best = min(best, e0.elapsed_time(e1))
+        return best
+    copy_ms = best_ms(lambda: dst.copy_(src), 5)
+    mm_ms = best_ms(lambda: torch.mm(a, b.t()), 5)
+    return {"copy_GBps": round(2 * src.numel() * 2 / copy_ms / 1e6, 1),
+            "gemm_TFLOPs": round(2 * n ** 3 / mm_ms / 1e9, 1)}
+
+
 def bench_workload(args) -> int:
     """A serving-style run: many concurrent requests through the scheduler (continuous batching,
     chunked prefill), as in the 14B and 32B workloads: ``--requests`` prompts of uniform random
@@ -245,6 +275,7 @@ def main() -> int:
             k = max(8, args.steps // 2)
             points[f"decode_b{b}"] = round(bench_decode(llm, b, args.context, k, 4, args.seed + 3 + b)["tok_s"], 1)
 
+    machine = measure_machine(torch.bfloat16 if elem == 2 else torch.float32)
     step_s = main_run["ms_per_step"] / 1e3
     achieved = decode_bytes(cfg, args.batch, int(main_run["mean_context"]), elem) / step_s / 1e9
     flops = prefill_flops(cfg, args.prefill_tokens)
@@ -271,10 +302,13 @@ def main() -> int:
             "decode_graph_replays": main_run["graph_replays"], "mean_context": round(main_run["mean_context"], 1),
         },
         "prefill": {"value": round(pre["tok_s"], 1), "tokens": args.prefill_tokens, "ms": round(pre["s"] * 1e3, 3),
-                    "frac": round(flops / pre["s"] / PEAK_FLOPS[dtype_key], 4)},
+                    "frac": round(flops / pre["s"] / PEAK_FLOPS[dtype_key], 4),
+                    "frac_of_measured_gemm": round(flops / pre["s"] / (machine["gemm_TFLOPs"] * 1e12), 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_GBPS, 4)},
+                     "frac": round(achieved / HBM_GBPS, 4),
+                     "frac_of_measured_copy": round(achieved / machine["copy_GBps"], 4)},
         "points": points,
+        "machine": machine,
     }
     print(json.dumps(line))
     torch.cuda.synchronize()
