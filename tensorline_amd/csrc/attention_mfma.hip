@@ -591,38 +591,95 @@ static size_t at_lds_bytes(int DC, int pages, int S) {
 }
 
 // Merge the splits of one (token, head): M = max m_s, out = sum acc_s e^(m_s - M) / sum l_s e^(m_s - M),
-// over the splits that hold keys of the token, in ascending order.
+// over the splits that hold keys of the token.  One work-group of 128 or 256 threads: a thread per split for
+// the weights, and (a float4 of the head, a group of splits) per thread for the sum, whose first eight
+// loads are in flight while the weights are found.
 #define AM_MAX_SPLITS 1024
-__global__ void attn_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
-                                  const int32_t* __restrict__ pos, bf16_t* __restrict__ out, int out_stride, int nq,
-                                  int D, int nsplit, int split_blocks, int window) {
+#define AM_MERGE_AHEAD 8
+template <int AM_MERGE_THREADS>
+__global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
+    const float* __restrict__ ws_o, const float* __restrict__ ws_ml, const int32_t* __restrict__ pos,
+    bf16_t* __restrict__ out, int out_stride, int nq, int D, int nsplit, int split_blocks, int window) {
     __shared__ float wgt[AM_MAX_SPLITS];
-    __shared__ float inv_l;
-    const int t = blockIdx.x, h = blockIdx.y;
+    __shared__ float red_m[AM_MERGE_THREADS / 64], red_l[AM_MERGE_THREADS / 64];
+    __shared__ float4 part[AM_MERGE_THREADS];
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int s_lo = (lo >> 5) / split_blocks, s_hi = (p >> 5) / split_blocks;
     const int ns = s_hi - s_lo + 1;
     const size_t base = ((size_t)t * nq + h) * nsplit + s_lo;
-    // every thread finds the maximum (a few cached loads), one thread per split its weight
-    float M = -INFINITY;
-    for (int s = 0; s < ns; ++s) M = fmaxf(M, ws_ml[(base + s) * 2]);
-    for (int s = threadIdx.x; s < ns; s += blockDim.x) {
-        const float ms = ws_ml[(base + s) * 2];
-        wgt[s] = (ms > -INFINITY) ? exp2f(ms - M) : 0.f;      // maxima are kept in the base-2 domain
+    const int D4 = D >> 2, SG = AM_MERGE_THREADS / D4;      // D is 32, 64 or 128
+    const int d4 = tid % D4, sg = tid / D4;
+    const float4* acc4 = reinterpret_cast<const float4*>(ws_o) + base * D4 + d4;
+    const float2* ml2 = reinterpret_cast<const float2*>(ws_ml) + base;
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 a[AM_MERGE_AHEAD];
+#pragma unroll
+    for (int k = 0; k < AM_MERGE_AHEAD; ++k) {
+        const int s = sg + k * SG;
+        a[k] = zero4;
+        if (s < ns) a[k] = acc4[(size_t)s * D4];
     }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        float L = 0.f;
-        for (int s = 0; s < ns; ++s) L += ws_ml[(base + s) * 2 + 1] * wgt[s];
-        inv_l = 1.0f / L;
+    float2 ml[AM_MAX_SPLITS / AM_MERGE_THREADS];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < AM_MAX_SPLITS / AM_MERGE_THREADS; ++j) {
+        const int s = tid + j * AM_MERGE_THREADS;
+        ml[j] = make_float2(-INFINITY, 0.f);
+        if (s < ns) ml[j] = ml2[s];
+        mx = fmaxf(mx, ml[j].x);
     }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if ((tid & 63) == 0) red_m[tid >> 6] = mx;
     __syncthreads();
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float o = 0.f;
-#pragma unroll 8
-        for (int s = 0; s < ns; ++s) o += ws_o[(base + s) * D + d] * wgt[s];
-        out[(size_t)t * out_stride + (size_t)h * D + d] = tl_from_float<bf16_t>(o * inv_l);
+    float M = red_m[0];
+#pragma unroll
+    for (int w = 1; w < AM_MERGE_THREADS / 64; ++w) M = fmaxf(M, red_m[w]);
+    float ls = 0.f;                                          // maxima are kept in the base-2 domain
+#pragma unroll
+    for (int j = 0; j < AM_MAX_SPLITS / AM_MERGE_THREADS; ++j) {
+        const int s = tid + j * AM_MERGE_THREADS;
+        const float w = (ml[j].x > -INFINITY) ? exp2f(ml[j].x - M) : 0.f;
+        if (s < ns) wgt[s] = w;
+        ls += ml[j].y * w;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ls += __shfl_xor(ls, o);
+    if ((tid & 63) == 0) red_l[tid >> 6] = ls;
+    __syncthreads();
+    float L = red_l[0];
+#pragma unroll
+    for (int w = 1; w < AM_MERGE_THREADS / 64; ++w) L += red_l[w];
+    float4 o4 = zero4;
+#pragma unroll
+    for (int k = 0; k < AM_MERGE_AHEAD; ++k) {
+        const int s = sg + k * SG;
+        if (s < ns) {
+            const float w = wgt[s];
+            o4.x += a[k].x * w, o4.y += a[k].y * w, o4.z += a[k].z * w, o4.w += a[k].w * w;
+        }
+    }
+    for (int s = sg + AM_MERGE_AHEAD * SG; s < ns; s += SG) {
+        const float4 v = acc4[(size_t)s * D4];
+        const float w = wgt[s];
+        o4.x += v.x * w, o4.y += v.y * w, o4.z += v.z * w, o4.w += v.w * w;
+    }
+    part[tid] = o4;
+    __syncthreads();
+    if (tid < D4) {
+        float4 r = part[tid];
+        for (int g = 1; g < SG; ++g) {
+            const float4 v = part[g * D4 + tid];
+            r.x += v.x, r.y += v.y, r.z += v.z, r.w += v.w;
+        }
+        const float inv_l = 1.0f / L;
+        bf16_t* dst = out + (size_t)t * out_stride + (size_t)h * D + tid * 4;
+        dst[0] = tl_from_float<bf16_t>(r.x * inv_l);
+        dst[1] = tl_from_float<bf16_t>(r.y * inv_l);
+        dst[2] = tl_from_float<bf16_t>(r.z * inv_l);
+        dst[3] = tl_from_float<bf16_t>(r.w * inv_l);
     }
 }
 
@@ -671,6 +728,8 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
                  "tl_attention_mfma: bad row strides %d, %d", q_stride, out_stride);
     TL_CHECK_ARG(((uintptr_t)q % 16) == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0 &&
                      ((uintptr_t)out % 8) == 0, "tl_attention_mfma: operands must be 16-byte aligned");
+    TL_CHECK_ARG(nsplit == 1 || (((uintptr_t)ws_o % 16) == 0 && ((uintptr_t)ws_ml % 8) == 0),
+                 "tl_attention_mfma: the split workspace must be 16-byte aligned");
     TL_CHECK_ARG(nkv <= 65535, "tl_attention_mfma: too many key/value heads");
     if (T == 0 || S == 0) return 0;
     const long waves = (long)max_tile_groups * nsplit;
@@ -707,8 +766,12 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
                        ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
     TL_CHECK_LAUNCH("tl_attention_mfma");
     if (nsplit > 1) {
-        hipLaunchKernelGGL(attn_merge_kernel, dim3(T, nq), dim3(d < 64 ? 64 : d), 0, stream, ws_o, ws_ml, pos,
-                           (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window);
+        if (nsplit > 32)
+            hipLaunchKernelGGL(attn_merge_kernel<256>, dim3(T, nq), dim3(256), 0, stream, ws_o, ws_ml, pos,
+                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window);
+        else
+            hipLaunchKernelGGL(attn_merge_kernel<128>, dim3(T, nq), dim3(128), 0, stream, ws_o, ws_ml, pos,
+                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window);
         TL_CHECK_LAUNCH("tl_attention_mfma merge");
     }
     return 0;
