@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int s = blockIdx.x, kvh = blockIdx.y;
-    const int widx = blockIdx.z * 4 + wave;
+    const int widx = blockIdx.z * (blockDim.x >> 6) + wave;    // one to four waves per work-group
     const int tg = widx / nsplit, sp = widx - tg * nsplit;
     const int G = nq / nkv;
     const float scale2 = scale * AM_LOG2E;
@@ -684,7 +684,7 @@ __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
 }
 
 template <int DC>
-static void launch_attn(int NT, dim3 grid, hipStream_t stream, const bf16_t* q, int q_stride, const bf16_t* kc,
+static void launch_attn(int NT, dim3 grid, int wg_waves, hipStream_t stream, const bf16_t* q, int q_stride, const bf16_t* kc,
                         const bf16_t* vc, const int32_t* tables, int NB, const int32_t* q_start,
                         const int32_t* ctx_start, bf16_t* out, int out_stride, float* ws_o, float* ws_ml, int nq, int nkv,
                         int bs, int window, float scale, int nsplit, int split_blocks) {
@@ -692,11 +692,11 @@ static void launch_attn(int NT, dim3 grid, hipStream_t stream, const bf16_t* q, 
     if ((bs & (bs - 1)) == 0)
         for (bs_shift = 0; (1 << bs_shift) < bs;) ++bs_shift;
     if (NT == 1)
-        hipLaunchKernelGGL((attn_mfma_kernel<DC, 1>), grid, dim3(256), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
+        hipLaunchKernelGGL((attn_mfma_kernel<DC, 1>), grid, dim3(64 * wg_waves), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
                            ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
                            split_blocks);
     else
-        hipLaunchKernelGGL((attn_mfma_kernel<DC, 2>), grid, dim3(256), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
+        hipLaunchKernelGGL((attn_mfma_kernel<DC, 2>), grid, dim3(64 * wg_waves), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
                            ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
                            split_blocks);
 }
@@ -733,8 +733,11 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     TL_CHECK_ARG(nkv <= 65535, "tl_attention_mfma: too many key/value heads");
     if (T == 0 || S == 0) return 0;
     const long waves = (long)max_tile_groups * nsplit;
-    TL_CHECK_ARG((waves + 3) / 4 <= 65535, "tl_attention_mfma: too many tile groups x splits (%ld)", waves);
-    dim3 grid(S, nkv, (unsigned)((waves + 3) / 4));
+    // The waves are independent: four to a work-group, fewer when that would leave compute units without one.
+    int wg_waves = 4;
+    while (wg_waves > 1 && (long)S * nkv * ((waves + wg_waves - 1) / wg_waves) < 256) wg_waves >>= 1;
+    TL_CHECK_ARG((waves + wg_waves - 1) / wg_waves <= 65535, "tl_attention_mfma: too many tile groups x splits (%ld)", waves);
+    dim3 grid(S, nkv, (unsigned)((waves + wg_waves - 1) / wg_waves));
     const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
     const bool pow2 = (bs & (bs - 1)) == 0;
     if (NT == 2 && nsplit == 1 && shared && pow2 && total_groups128 > 0 && at_lds_bytes(d / 32, NB, S) <= 160 * 1024) {
@@ -756,13 +759,13 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
         return 0;
     }
     if (d == 32)
-        launch_attn<1>(NT, grid, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
+        launch_attn<1>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
                        ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
     else if (d == 64)
-        launch_attn<2>(NT, grid, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
+        launch_attn<2>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
                        ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
     else
-        launch_attn<4>(NT, grid, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
+        launch_attn<4>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
                        ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
     TL_CHECK_LAUNCH("tl_attention_mfma");
     if (nsplit > 1) {
