@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import threading
+import warnings
 from dataclasses import dataclass
 
 import torch
@@ -384,6 +385,9 @@ def tune_library_linear(rows: int, weight: torch.Tensor, out_dtype: torch.dtype,
     try:
         _library_linear(a, weight, None, out_dtype)
         torch.cuda.synchronize(weight.device)
+    except RuntimeError as e:                            # the search is optional: the heuristic choice stays
+        warnings.warn(f"library tuning of the {tuple(weight.shape)} product failed and is skipped: {e}")
+        return False
     finally:
         tn.tuning_enable(False)
     return True
