@@ -6,7 +6,11 @@ library, a tensor that is not on the GPU or a size a kernel does not take raises
 """
 from __future__ import annotations
 
+import atexit
 import ctypes
+import glob
+import os
+import tempfile
 import threading
 import warnings
 from dataclasses import dataclass
@@ -363,6 +367,30 @@ def _library_linear(a, weight, bias, out_dtype) -> torch.Tensor:
     return y
 
 
+_TUNING_RECORD: str | None = None
+
+
+def _keep_tuning_records_out_of_the_way(tn) -> None:
+    """TunableOp records what it finds in a file, by default in the working directory: the record
+    goes to a file of this process in the temporary directory instead and is removed at exit (a
+    search is repeated in every process; nothing is read back)."""
+    global _TUNING_RECORD
+    if _TUNING_RECORD is not None:
+        return
+    if hasattr(tn, "write_file_on_exit"):
+        tn.write_file_on_exit(False)
+    _TUNING_RECORD = os.path.join(tempfile.gettempdir(), f"tensorline_amd_tuning_{os.getuid()}_{os.getpid()}.csv")
+    tn.set_filename(_TUNING_RECORD)
+
+    def remove():
+        for path in glob.glob(_TUNING_RECORD[:-4] + "*"):
+            try:
+                os.remove(path)
+            except OSError:
+                pass
+    atexit.register(remove)
+
+
 def tune_library_linear(rows: int, weight: torch.Tensor, out_dtype: torch.dtype, seconds: float = 2.0) -> bool:
     """Have the library pick its kernel for the ``[rows, K] x [N, K]^T`` product by measurement
     (torch's TunableOp searches the hipBLASLt and rocBLAS solutions once and keeps the fastest for
@@ -376,8 +404,7 @@ def tune_library_linear(rows: int, weight: torch.Tensor, out_dtype: torch.dtype,
         return False
     _on_gpu(weight)
     tn.enable(True)
-    if hasattr(tn, "write_file_on_exit"):
-        tn.write_file_on_exit(False)
+    _keep_tuning_records_out_of_the_way(tn)
     tn.set_max_tuning_duration(int(seconds * 1000))
     tn.set_max_tuning_iterations(50)
     a = torch.randn(rows, weight.shape[1], device=weight.device).to(torch.bfloat16)
