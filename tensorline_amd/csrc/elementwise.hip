@@ -217,7 +217,7 @@ template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict__ pos,
                                   const float* __restrict__ inv_freq, T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   const int32_t* __restrict__ slots, int nq, int nkv, int d, int rot, int write_kv,
-                                  int bs, const float* __restrict__ bias) {
+                                  int bs, const float* __restrict__ bias, int vec8) {
     __shared__ float cs_s[256], sn_s[256];          // one sine and cosine per rotated pair of the token
     const int t = blockIdx.x;
     const int half = rot / 2;
@@ -227,7 +227,40 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
     const int nrot = nq + nkv;  // heads that are rotated: q then k
     for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(p * inv_freq[i], &sn_s[i], &cs_s[i]);
     __syncthreads();
-    // rotated pairs
+    // rotated pairs; bfloat16 with eight pairs to a thread where the sizes allow 16-byte accesses
+    if (vec8) {
+        if constexpr (sizeof(T) == 2) {
+            const int per_head = half >> 3;
+            for (int idx = threadIdx.x; idx < nrot * per_head; idx += blockDim.x) {
+                const int h = idx / per_head, i = (idx - h * per_head) * 8;
+                bf16_t* hp = reinterpret_cast<bf16_t*>(row) + (size_t)h * d;
+                const uint4 lo = *reinterpret_cast<const uint4*>(hp + i);
+                const uint4 hi = *reinterpret_cast<const uint4*>(hp + i + half);
+                const uint32_t lw[4] = {lo.x, lo.y, lo.z, lo.w}, hw[4] = {hi.x, hi.y, hi.z, hi.w};
+                uint32_t o1[4], o2[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    float a0 = __uint_as_float(lw[k] << 16), a1 = __uint_as_float(lw[k] & 0xffff0000u);
+                    float b0 = __uint_as_float(hw[k] << 16), b1 = __uint_as_float(hw[k] & 0xffff0000u);
+                    if (bias) {
+                        a0 += bias[h * d + i + 2 * k], a1 += bias[h * d + i + 2 * k + 1];
+                        b0 += bias[h * d + i + half + 2 * k], b1 += bias[h * d + i + half + 2 * k + 1];
+                    }
+                    const float c0 = cs_s[i + 2 * k], c1 = cs_s[i + 2 * k + 1];
+                    const float s0 = sn_s[i + 2 * k], s1 = sn_s[i + 2 * k + 1];
+                    o1[k] = (uint32_t)tl_f2bf_bits(a0 * c0 - b0 * s0) | ((uint32_t)tl_f2bf_bits(a1 * c1 - b1 * s1) << 16);
+                    o2[k] = (uint32_t)tl_f2bf_bits(b0 * c0 + a0 * s0) | ((uint32_t)tl_f2bf_bits(b1 * c1 + a1 * s1) << 16);
+                }
+                bf16_t* dst = hp;
+                if (h >= nq) {
+                    if (slot < 0) continue;
+                    dst = reinterpret_cast<bf16_t*>(k_cache) + ((size_t)slot * nkv + (h - nq)) * d;
+                }
+                *reinterpret_cast<uint4*>(dst + i) = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+                *reinterpret_cast<uint4*>(dst + i + half) = make_uint4(o2[0], o2[1], o2[2], o2[3]);
+            }
+        }
+    } else
     for (int idx = threadIdx.x; idx < nrot * half; idx += blockDim.x) {
         const int h = idx / half, i = idx - h * half;
         const float sn = sn_s[i], cs = cs_s[i];
@@ -280,12 +313,15 @@ extern "C" int tl_rope_store(void* qkv, int dtype, const int32_t* pos, const flo
     TL_CHECK_ARG(!write_kv || (k_cache && v_cache && slots && bs > 0), "tl_rope_store: cache write asked for without a cache");
     if (T == 0) return 0;
     dim3 grid(T), block(256);
+    // 16-byte accesses: every head and both halves of the rotated part start at a multiple of 8 values
+    const int vec8 = dtype == TL_BF16 && d % 8 == 0 && rot % 16 == 0 && rot > 0 && ((uintptr_t)qkv % 16) == 0 &&
+                     (!write_kv || ((uintptr_t)k_cache % 16) == 0);
     if (dtype == TL_F32)
         hipLaunchKernelGGL(rope_store_kernel<float>, grid, block, 0, stream, (float*)qkv, pos, inv_freq,
-                           (float*)k_cache, (float*)v_cache, slots, nq, nkv, d, rot, write_kv, bs, bias);
+                           (float*)k_cache, (float*)v_cache, slots, nq, nkv, d, rot, write_kv, bs, bias, 0);
     else if (dtype == TL_BF16)
         hipLaunchKernelGGL(rope_store_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, pos, inv_freq,
-                           (bf16_t*)k_cache, (bf16_t*)v_cache, slots, nq, nkv, d, rot, write_kv, bs, bias);
+                           (bf16_t*)k_cache, (bf16_t*)v_cache, slots, nq, nkv, d, rot, write_kv, bs, bias, vec8);
     else
         return tl_fail("tl_rope_store: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("tl_rope_store");
