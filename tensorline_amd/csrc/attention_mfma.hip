@@ -280,25 +280,28 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     }
 }
 
-// The same block of 32 keys with the fragments taken from LDS where they are used: kt points at
-// the block's 32 key rows (KP units each) in matrix-core order (row c of score tile 0, which is key
-// 8 (c / 4) + c % 4, in LDS row c, row c of tile 1 in LDS row 16 + c: the 16 lanes of a read then
-// take 16 consecutive rows, which the one unit of padding spreads over all banks), vt at the
-// block's 4 units of dim row 0 (VP units per dim).  All score tiles first, then the softmax of each column tile, then all P*V products, so
-// that key fragments are dead before value fragments are read: few registers are live at once.
-template <int DC, int NT, int KP, int VP>
-__device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, const uint4 (*qf)[DC], const int* p_col,
-                                             const int* lo_col, int kb, int c, int g, float scale2, float* m_run,
-                                             float* l_run, f32x4 (*acc)[DC * 2]) {
+// The same block of 32 keys (half `half` of a 64-key tile) with the fragments taken from LDS where
+// they are used.  kt is the tile's 64 key rows of 4 DC units in matrix-core order (row c of score
+// tile r, which is key 32 (r / 2) + 8 (c / 4) + 4 (r % 2) + c % 4 of the tile, in LDS row 16 r + c), vt
+// its 32 DC dim rows of 8 units (8 keys each).  Rows are not padded: unit u of a row lies at u ^ kx
+// (keys) or u ^ vx (values), kx and vx depending on the row so that the 16 lanes of a read, which
+// take the same unit of 16 consecutive rows, are spread over all banks (at_k_swizzle, at_v_swizzle).
+// All score tiles first, then the softmax of each column tile, then all P*V products, so that key
+// fragments are dead before value fragments are read: few registers are live at once.
+template <int DC, int NT>
+__device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, int kx, int vx, int half,
+                                             const uint4 (*qf)[DC], const int* p_col, const int* lo_col, int kb, int c,
+                                             int g, float scale2, float* m_run, float* l_run, f32x4 (*acc)[DC * 2]) {
     constexpr int DB = DC * 2;
+    constexpr int UPK = DC * 4;
     const int key_base = kb + 8 * g;
     f32x4 st0[NT], st1[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) st0[j] = st1[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int dc = 0; dc < DC; ++dc) {
-        const uint4 k0 = kt[c * KP + dc * 4 + g];
-        const uint4 k1 = kt[(16 + c) * KP + dc * 4 + g];
+        const uint4 k0 = kt[(32 * half + c) * UPK + ((dc * 4 + g) ^ kx)];
+        const uint4 k1 = kt[(32 * half + 16 + c) * UPK + ((dc * 4 + g) ^ kx)];
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
             st0[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(k0), am_frag(qf[j][dc]), st0[j], 0, 0, 0);
@@ -359,35 +362,176 @@ __device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, c
     }
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-        const uint4 v = vt[(db * 16 + c) * VP + g];
+        const uint4 v = vt[(db * 16 + c) * 8 + ((4 * half + g) ^ vx)];
 #pragma unroll
         for (int j = 0; j < NT; ++j)
             acc[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(v), am_frag(pf[j]), acc[j][db], 0, 0, 0);
     }
 }
 
+// max(a, b, c) of numbers that are not NaN as the one instruction it is (fmaxf first quiets each
+// operand with an instruction of its own)
+__device__ __forceinline__ float am_max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// The maximum over the four lanes that hold one column (lanes c, c + 16, c + 32, c + 48), in all
+// four: two swaps of 16- and 32-lane halves between registers instead of two trips through LDS.
+typedef unsigned int am_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float am_column_max(float v) {
+    am_u32x2 sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = am_max3(v, __uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return am_max3(v, __uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+
+// A whole tile of 64 keys for one column tile of a wave, all of whose keys some column of the wave
+// sees: the same arithmetic as two calls of am_block_lds with one softmax step instead of two (one
+// maximum, one decision to move the running maximum), the scale folded into the exponent's
+// argument, and the LDS reads ahead of the products that use them: the key fragments of two
+// 32-wide slices of the head are in flight while the products of the slice before run, the value
+// fragments of the first 32 keys while the softmax is computed.
+template <int DC>
+__device__ __forceinline__ void am_tile_lds(const uint4* kt, const uint4* vt, int kx, int vx, const uint4* qf,
+                                            int p_col, int lo_col, int kb, int c, int g, float scale2, float& m_run,
+                                            float& l_run, f32x4* acc) {
+    constexpr int DB = DC * 2;
+    constexpr int UPK = DC * 4;
+    f32x4 st[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) st[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+    {
+        // a ring of four fragments: each is replaced, right behind the product that used it, by
+        // the one needed four products later
+        uint4 kf[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) kf[r] = kt[(16 * r + c) * UPK + (g ^ kx)];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                st[r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(kf[r]), am_frag(qf[dc]), st[r], 0, 0, 0);
+                if (dc + 1 < DC) kf[r] = kt[(16 * r + c) * UPK + (((dc + 1) * 4 + g) ^ kx)];
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    // The value fragments in the order of their products: those of the first 32 keys for every 16
+    // dims, then those of the last 32.  The first four are on their way during the softmax.
+    uint4 vf[4];
+#define AM_VFRAG(I) vt[((((I) % DB) * 16 + c) * 8) + ((4 * ((I) / DB) + g) ^ vx)]
+#pragma unroll
+    for (int i = 0; i < 4; ++i) vf[i] = AM_VFRAG(i);
+    __builtin_amdgcn_sched_barrier(0);
+    // lane (c, g) holds, of column c, keys kb + 32 h + 8 g + 4 r + i in st[2 h + r][i]
+    float sv[16];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sv[4 * r + i] = st[r][i];
+    const bool edge = (kb + 63 > p_col) || (kb < lo_col);
+    if (__any(edge)) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int key = kb + 32 * h + 8 * g + i;
+                if (key > p_col || key < lo_col) sv[8 * h + i] = -INFINITY;
+            }
+    }
+    float bmax = am_max3(am_max3(am_max3(sv[0], sv[1], sv[2]), am_max3(sv[3], sv[4], sv[5]), sv[6]),
+                         am_max3(am_max3(sv[7], sv[8], sv[9]), am_max3(sv[10], sv[11], sv[12]), sv[13]), am_max3(sv[14], sv[15], sv[15]));
+    bmax = am_column_max(bmax);
+    bmax *= scale2;                                          // the scale is positive: the order is the same
+    const bool moved = bmax > m_run + AM_LAZY || (m_run == -INFINITY && bmax > -INFINITY);
+    const float m_new = moved ? bmax : m_run;
+    const float neg_m = (m_new == -INFINITY) ? 0.f : -m_new;
+    float pr[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) pr[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[i], scale2, neg_m));
+    const float psum = (((pr[0] + pr[1]) + (pr[2] + pr[3])) + ((pr[4] + pr[5]) + (pr[6] + pr[7]))) +
+                       (((pr[8] + pr[9]) + (pr[10] + pr[11])) + ((pr[12] + pr[13]) + (pr[14] + pr[15])));
+    uint4 pf[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        pf[h].x = am_pack2(pr[8 * h + 0], pr[8 * h + 1]);
+        pf[h].y = am_pack2(pr[8 * h + 2], pr[8 * h + 3]);
+        pf[h].z = am_pack2(pr[8 * h + 4], pr[8 * h + 5]);
+        pf[h].w = am_pack2(pr[8 * h + 6], pr[8 * h + 7]);
+    }
+    if (__any(moved)) {
+        const float alpha = __builtin_amdgcn_exp2f(m_run + neg_m);
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            acc[db][0] *= alpha;
+            acc[db][1] *= alpha;
+            acc[db][2] *= alpha;
+            acc[db][3] *= alpha;
+        }
+    } else {
+        l_run += psum;
+    }
+    m_run = m_new;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 2 * DB; ++i) {
+        acc[i % DB] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(vf[i % 4]), am_frag(pf[i / DB]), acc[i % DB], 0, 0, 0);
+        if (i + 4 < 2 * DB) vf[i % 4] = AM_VFRAG(i + 4);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#undef AM_VFRAG
+}
+
 // The kernel for steps with prompt portions.  A work-group owns 128 consecutive columns of one
 // (sequence, key/value head), 16 * NT per wave, and walks the keys together in tiles of 64.  A
-// tile is brought into LDS once, with contiguous loads (whole key rows of K, runs of keys of one
-// dim of V^T), and every wave takes its MFMA fragments from there: keys and values are read from
-// the cache once per 128 columns, and a wave holds no copy of them in registers, so two
-// work-groups (sixteen waves) fit on a CU and some compute while others wait.  Two LDS buffers:
-// the loads of tile t + 1 are in flight (in registers) while tile t is multiplied, and go to the
-// other buffer before the one barrier of the iteration.  The sequence's page ids are copied to
-// LDS first, so a tile's addresses depend on no load from memory.  Pages must hold a power of two
-// of tokens (at least 8; 2^bs_shift): an 8-key run of V^T then lies in one page and a page id is
-// a shift away.  No key split: a step with prompt portions has columns enough.  (Measured on a
-// 2,048-token prompt at 28/4 heads of 128: 86 us with one column tile on each of eight waves, 98 us
-// with two on each of four; the time is that of the last group, which walks all the keys.)
+// tile is brought into LDS once and every wave takes its MFMA fragments from there: keys and
+// values are read from the cache once per 128 columns, and a wave holds no copy of them in
+// registers, so two work-groups (sixteen waves) fit on a CU and some compute while others wait.
+// The tile goes from memory straight into LDS (global_load_lds_dwordx4: each lane brings 16 bytes,
+// a wave's 64 lanes fill 1 KB of consecutive LDS), so it passes through no registers either: which
+// 16 bytes a lane asks for is chosen so that the consecutive LDS image is the swizzled layout the
+// fragment reads expect.  Two LDS buffers: the loads of tile t + 1 are in flight while tile t is
+// multiplied; every wave waits for its own loads before the one barrier of the iteration.  The
+// sequence's page ids are copied to LDS first, so a tile's addresses depend on no load from
+// memory.  Pages must hold a power of two of tokens (at least 8; 2^bs_shift): an 8-key run of V^T
+// then lies in one page and a page id is a shift away.  No key split: a step with prompt portions
+// has columns enough.
 #define AT_KEYS 64
 #define AT_NT 1                      // column tiles per wave; 8 / AT_NT waves in a work-group
-// LDS row of key k of a tile (see am_block_lds)
+// LDS row of key k of a tile (see am_block_lds), and the key of an LDS row
 __device__ __forceinline__ int at_lds_row(int k) {
     return (k & 32) + ((k & 4) << 2) + ((k & 24) >> 1) + (k & 3);
 }
+__device__ __forceinline__ int at_lds_key(int row) {
+    return (row & 35) + ((row & 16) >> 2) + ((row & 12) << 1);
+}
+// Where unit u of a row lies in it: u ^ swizzle(row).  A K row has UPK = 4, 8 or 16 units, so 16 /
+// UPK rows span the 256 bytes over which the banks repeat; the swizzle steps once per such span.  A
+// V^T row has 8 units.  Both depend only on the row modulo 16 (the lane's c in a fragment read).
+template <int UPK>
+__device__ __forceinline__ int at_k_swizzle(int row) { return ((row & 15) * UPK) >> 4; }
+__device__ __forceinline__ int at_v_swizzle(int row) { return (row >> 1) & 7; }
+
+// 16 bytes per lane from memory straight into LDS at lds_base + 16 * lane (lds_base is the same for
+// the whole wave).  Written as assembly so that the compiler does not make every later LDS read wait
+// for it: a load is waited for only where AT_LANDED says so.  M0 holds the LDS base for the
+// instruction and is put back.
+__device__ __forceinline__ void at_load_to_lds(const void* g, void* lds_base) {
+    const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds_base;
+    uint32_t saved;
+    asm volatile(
+        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+        : "=&s"(saved)
+        : "s"(base), "v"(g)
+        : "memory");
+}
 
 template <int DC, int NT, int WAVES>
-__global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
+__global__ __launch_bounds__(WAVES * 64, 32 / WAVES) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int S, int nq, int nkv, int bs,
@@ -396,12 +540,12 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
     constexpr int WCOLS = NT * 16;                       // columns of a wave; WAVES * WCOLS = 128 per work-group
     constexpr int D = DC * 32;
     constexpr int DB = D / 16;
-    constexpr int KP = D / 8 + 1;             // uint4 per key row in LDS (one of padding)
-    constexpr int VP = AT_KEYS / 8 + 1;       // uint4 per dim row in LDS: 64 keys + padding
+    constexpr int UPK = D / 8;                // uint4 per key row; also the wave-loads of a K tile and of a V^T tile
+    constexpr int TILE = AT_KEYS * UPK;       // uint4 of a K tile, and of a V^T tile (D rows of 8)
     extern __shared__ uint4 at_smem[];
-    uint4* ks = at_smem;                                   // [2][AT_KEYS * KP]
-    uint4* vs = at_smem + 2 * AT_KEYS * KP;                // [2][D * VP]
-    int* tab = reinterpret_cast<int*>(vs + 2 * D * VP);    // page ids of the sequence, as far as needed (NB ints)
+    uint4* ks = at_smem;                                   // [2][TILE]
+    uint4* vs = at_smem + 2 * TILE;                        // [2][TILE]
+    int* tab = reinterpret_cast<int*>(vs + 2 * TILE);      // page ids of the sequence, as far as needed (NB ints)
     int* qst = tab + NB;                                   // q_start of the step (S + 1 ints)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
@@ -425,28 +569,29 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
     const int n = qst[s + 1] - r0;
     const int start = ctx_start[s];
     const int ncols = n * G;
-    // Loader.  A K tile is 64 keys x D/8 units of 16 bytes, a V^T tile D dims x 8 units (8 keys
-    // each): LU units of each per thread (threads past the last unit repeat it and store nothing).
-    // K: consecutive threads take consecutive units of a key row.  V^T: consecutive threads take
-    // the units of one dim inside a page, then the next dim, which is how a page lies in memory
-    // ([dim][token]); `opp` units of a dim are in one page.
-    const int opp_shift = (bs_shift < 6) ? bs_shift - 3 : 3;    // log2(min(bs, 64) / 8)
-    constexpr int UPK = D / 8;                               // units per key row
-    constexpr int UNITS = AT_KEYS * UPK;                     // units of a K tile, and of a V^T tile
-    constexpr int LU = (UNITS + THREADS - 1) / THREADS;
-    int k_at[LU], v_at[LU];                                  // key | unit << 16;  dim | first key of the unit << 16
-    bool u_mine[LU];
+    // Loader.  A K tile is 64 rows x UPK units of 16 bytes, a V^T tile D rows x 8 units (8 keys
+    // each): UPK wave-loads of 64 consecutive units each, dealt round-robin to the waves.  For its
+    // load number i a lane knows which key and unit (K) and which dim and first key (V^T) the LDS
+    // place it fills holds.
+    constexpr int NI = (UPK + WAVES - 1) / WAVES;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    int k_key[NI], v_key[NI];                  // K: the lane's key of the tile; V^T: the first key of its unit
+    const char *k_base[NI], *v_base[NI];       // where that unit lies in slot 0 (K), in page 0 at offset 0 (V^T)
 #pragma unroll
-    for (int i = 0; i < LU; ++i) {
-        int u = tid + THREADS * i;
-        u_mine[i] = u < UNITS;
-        if (!u_mine[i]) u = UNITS - 1;
-        k_at[i] = (u / UPK) | ((u % UPK) << 16);
-        const int o = u & ((1 << opp_shift) - 1);
-        const int rest = u >> opp_shift;
-        v_at[i] = (rest % D) | (((((rest / D) << opp_shift) + o) * 8) << 16);
+    for (int i = 0; i < NI; ++i) {
+        int w = wave_u + i * WAVES;
+        if (w >= UPK) w = UPK - 1;                           // not issued
+        const int idx = w * 64 + lane;
+        const int krow = idx / UPK, kpu = idx % UPK;
+        k_key[i] = at_lds_key(krow);
+        k_base[i] = reinterpret_cast<const char*>(kc + (size_t)kvh * D + (kpu ^ at_k_swizzle<UPK>(krow)) * 8);
+        const int vrow = idx >> 3, vpu = idx & 7;
+        v_key[i] = (vpu ^ at_v_swizzle(vrow)) * 8;
+        v_base[i] = reinterpret_cast<const char*>(vc + ((size_t)kvh * D + vrow) * bs);
     }
-    uint4 kreg[LU], vreg[LU];
+    const uint32_t k_stride = (uint32_t)nkv * D * 2;         // bytes from a slot to the next
+    const uint32_t v_stride = (uint32_t)nkv * D * bs * 2;    // bytes from a page to the next
+    const int kx = at_k_swizzle<UPK>(c), vx = at_v_swizzle(c);
     const int wg_col0 = (ngroups - 1 - flat) * 128;
     const int col0 = wg_col0 + wave * WCOLS;
     const bool wave_active = col0 < ncols;
@@ -507,54 +652,55 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
         for (int db = 0; db < DB; ++db) acc[j][db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-#define AT_PAGE(KEY, PG, OFF)                                                                                  \
-    OFF = (KEY) & (bs - 1);                                                                                   \
-    PG = tab[(KEY) >> bs_shift];
-#define AT_FETCH(T)                                                                                            \
+    // Tile T into buffer BUF: nothing comes back into registers.  All addresses first (their page
+    // ids come from LDS), then the loads.  A key past the last one any column sees is masked for
+    // every column: it is read from the last key's place, which stays on pages the sequence owns.
+#define AT_FETCH(T, BUF)                                                                                       \
     {                                                                                                         \
         const int kb_ = (T) * AT_KEYS;                                                                        \
-        _Pragma("unroll") for (int i = 0; i < LU; ++i) {                                                      \
-            int key_ = kb_ + (k_at[i] & 0xffff);                                                              \
-            if (key_ > khi) key_ = khi; /* masked for every column; stay on owned pages */                    \
-            int pg_, off_;                                                                                    \
-            AT_PAGE(key_, pg_, off_)                                                                          \
-            kreg[i] = *reinterpret_cast<const uint4*>(kc + ((size_t)(pg_ * bs + off_) * nkv + kvh) * D + (k_at[i] >> 16) * 8); \
-        }                                                                                                     \
-        _Pragma("unroll") for (int i = 0; i < LU; ++i) {                                                      \
-            int vk_ = kb_ + (v_at[i] >> 16);                                                                  \
+        const char *gk_[NI], *gv_[NI];                                                                        \
+        _Pragma("unroll") for (int i = 0; i < NI; ++i) {                                                      \
+            int key_ = kb_ + k_key[i];                                                                        \
+            if (key_ > khi) key_ = khi;                                                                       \
+            const uint32_t slot_ = ((uint32_t)tab[key_ >> bs_shift] << bs_shift) + (key_ & (bs - 1));         \
+            gk_[i] = k_base[i] + (uint64_t)slot_ * k_stride;                                                  \
+            int vk_ = kb_ + v_key[i];                                                                         \
             if (vk_ > khi) vk_ = khi & ~7;                                                                    \
-            int pg_, off_;                                                                                    \
-            AT_PAGE(vk_, pg_, off_)                                                                           \
-            vreg[i] = *reinterpret_cast<const uint4*>(vc + (((size_t)pg_ * nkv + kvh) * D + (v_at[i] & 0xffff)) * bs + off_); \
+            gv_[i] = v_base[i] + (uint64_t)(uint32_t)tab[vk_ >> bs_shift] * v_stride + (vk_ & (bs - 1)) * 2;  \
         }                                                                                                     \
-    }
-#define AT_STASH(BUF)                                                                                          \
-    {                                                                                                         \
-        _Pragma("unroll") for (int i = 0; i < LU; ++i) {                                                      \
-            if (u_mine[i]) {                                                                                  \
-                ks[(BUF) * AT_KEYS * KP + at_lds_row(k_at[i] & 0xffff) * KP + (k_at[i] >> 16)] = kreg[i];      \
-                vs[(BUF) * D * VP + (v_at[i] & 0xffff) * VP + (v_at[i] >> 19)] = vreg[i];                      \
+        _Pragma("unroll") for (int i = 0; i < NI; ++i) {                                                      \
+            const int w_ = wave_u + i * WAVES;                                                                \
+            if (w_ < UPK) {                                                                                   \
+                at_load_to_lds(gk_[i], ks + (BUF) * TILE + w_ * 64);                                          \
+                at_load_to_lds(gv_[i], vs + (BUF) * TILE + w_ * 64);                                          \
             }                                                                                                 \
         }                                                                                                     \
     }
+    // every load of this wave has landed (vmcnt 0; the other counters are left alone)
+#define AT_LANDED() __builtin_amdgcn_s_waitcnt(0x0f70)
 
     __syncthreads();                                         // the page ids are in LDS
-    AT_FETCH(t_lo)
-    AT_STASH(0)
+    AT_FETCH(t_lo, 0)
+    AT_LANDED();
     __syncthreads();
     int cur = 0;
     for (int t = t_lo; t <= t_hi; ++t) {
-        AT_FETCH(t < t_hi ? t + 1 : t)                       // past the last tile: the same again, unused
-        const uint4* kt = ks + cur * AT_KEYS * KP;
-        const uint4* vt = vs + cur * D * VP;
+        if (t < t_hi) AT_FETCH(t + 1, cur ^ 1)
+        const uint4* kt = ks + cur * TILE;
+        const uint4* vt = vs + cur * TILE;
+        if (NT == 1 && t * AT_KEYS + 32 <= wk_hi && t * AT_KEYS + 31 >= wk_lo) {
+            // both halves hold keys of the wave: the whole tile at once
+            am_tile_lds<DC>(kt, vt, kx, vx, qf[0], p_col[0], lo_col[0], t * AT_KEYS, c, g, scale2, m_run[0], l_run[0],
+                            acc[0]);
+        } else {
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int kb = t * AT_KEYS + half * 32;
-            if (kb > wk_hi || kb + 31 < wk_lo) continue;      // the same for the whole wave
-            am_block_lds<DC, NT, KP, VP>(kt + half * 32 * KP, vt + half * 4, qf, p_col, lo_col, kb, c, g, scale2, m_run,
-                                         l_run, acc);
+            for (int half = 0; half < 2; ++half) {
+                const int kb = t * AT_KEYS + half * 32;
+                if (kb > wk_hi || kb + 31 < wk_lo) continue;  // the same for the whole wave
+                am_block_lds<DC, NT>(kt, vt, kx, vx, half, qf, p_col, lo_col, kb, c, g, scale2, m_run, l_run, acc);
+            }
         }
-        AT_STASH(cur ^ 1)
+        AT_LANDED();
         __syncthreads();
         cur ^= 1;
     }
@@ -577,17 +723,14 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile_kernel(
     }
 }
 
-#undef AT_PAGE
 #undef AT_FETCH
-#undef AT_STASH
+#undef AT_LANDED
 
-// LDS of the tile kernel for head size 32 * DC, a table of `pages` page ids and S sequences: 70 KB of tiles at
-// head size 128, so two work-groups share a CU's 160 KB up to 2,560 pages per sequence and one
+// LDS of the tile kernel for head size 32 * DC, a table of `pages` page ids and S sequences: 64 KB of tiles at
+// head size 128, so two work-groups share a CU's 160 KB up to some 8,000 pages per sequence and one
 // work-group has it alone beyond that
 static size_t at_lds_bytes(int DC, int pages, int S) {
-    const int D = DC * 32;
-    return (size_t)(2 * AT_KEYS * (D / 8 + 1) + 2 * D * (AT_KEYS / 8 + 1)) * sizeof(uint4) +
-           (size_t)(pages + S + 1) * sizeof(int);
+    return (size_t)(4 * AT_KEYS * DC * 4) * sizeof(uint4) + (size_t)(pages + S + 1) * sizeof(int);
 }
 
 // Merge the splits of one (token, head): M = max m_s, out = sum acc_s e^(m_s - M) / sum l_s e^(m_s - M),
@@ -731,6 +874,7 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     TL_CHECK_ARG(nsplit == 1 || (((uintptr_t)ws_o % 16) == 0 && ((uintptr_t)ws_ml % 8) == 0),
                  "tl_attention_mfma: the split workspace must be 16-byte aligned");
     TL_CHECK_ARG(nkv <= 65535, "tl_attention_mfma: too many key/value heads");
+    TL_CHECK_ARG(scale > 0.f, "tl_attention_mfma: the score scale %g must be positive", (double)scale);
     if (T == 0 || S == 0) return 0;
     const long waves = (long)max_tile_groups * nsplit;
     // The waves are independent: four to a work-group, fewer when that would leave compute units without one.
