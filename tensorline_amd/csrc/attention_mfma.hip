@@ -43,6 +43,24 @@ __device__ __forceinline__ uint32_t am_pack2(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
+// max(a, b, c) of numbers that are not NaN as the one instruction it is (fmaxf first quiets each
+// operand with an instruction of its own)
+__device__ __forceinline__ float am_max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// The maximum over the four lanes that hold one column (lanes c, c + 16, c + 32, c + 48), in all
+// four: two swaps of 16- and 32-lane halves between registers instead of two trips through LDS.
+typedef unsigned int am_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float am_column_max(float v) {
+    am_u32x2 sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = am_max3(v, __uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return am_max3(v, __uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+
 #define AM_LOG2E 1.4426950408889634f
 #define AM_LAZY 8.0f                 // how far a block's maximum may exceed the running one before it moves
 #define AM_NO_COLUMN 0x7fffffff      // position of a lane without a column: never masks, never written
@@ -80,9 +98,7 @@ __device__ __forceinline__ void am_block(const uint4* kf0, const uint4* kf1, con
                 if (key > p_col[j] || key < lo_col[j]) sv[i] = -INFINITY;
             }
         }
-        float bmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 16, TL_WAVE));
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, TL_WAVE));
+        const float bmax = am_column_max(am_max3(am_max3(sv[0], sv[1], sv[2]), am_max3(sv[3], sv[4], sv[5]), am_max3(sv[6], sv[7], sv[7])));
         const float m_new = fmaxf(m_run[j], bmax);
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
         const bool moved = m_new > m_run[j];
@@ -325,9 +341,7 @@ __device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, i
                 if (key > p_col[j] || key < lo_col[j]) sv[i] = -INFINITY;
             }
         }
-        float bmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 16, TL_WAVE));
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, TL_WAVE));
+        const float bmax = am_column_max(am_max3(am_max3(sv[0], sv[1], sv[2]), am_max3(sv[3], sv[4], sv[5]), am_max3(sv[6], sv[7], sv[7])));
         // The running maximum follows the true one lazily: it moves only when the block's maximum
         // exceeds it by more than AM_LAZY (in the base-2 domain), so probabilities stay below
         // 2^AM_LAZY and the accumulator is rescaled in few blocks instead of most.  Sums and
@@ -367,24 +381,6 @@ __device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, i
         for (int j = 0; j < NT; ++j)
             acc[j][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am_frag(v), am_frag(pf[j]), acc[j][db], 0, 0, 0);
     }
-}
-
-// max(a, b, c) of numbers that are not NaN as the one instruction it is (fmaxf first quiets each
-// operand with an instruction of its own)
-__device__ __forceinline__ float am_max3(float a, float b, float c) {
-    float r;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
-
-// The maximum over the four lanes that hold one column (lanes c, c + 16, c + 32, c + 48), in all
-// four: two swaps of 16- and 32-lane halves between registers instead of two trips through LDS.
-typedef unsigned int am_u32x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ float am_column_max(float v) {
-    am_u32x2 sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    v = am_max3(v, __uint_as_float(sw[0]), __uint_as_float(sw[1]));
-    sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return am_max3(v, __uint_as_float(sw[0]), __uint_as_float(sw[1]));
 }
 
 // A whole tile of 64 keys for one column tile of a wave, all of whose keys some column of the wave
