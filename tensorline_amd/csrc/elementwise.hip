@@ -59,10 +59,13 @@ extern "C" int tl_embed(const int32_t* ids, const void* table, int table_dtype, 
 // ---- residual add + RMSNorm ----------------------------------------------------------------
 // Without `rows`: x[r] += residual[r] (written back, float), out[r] = x[r] * rstd * w.
 // With `rows`:    out[r] = norm(x[rows[r]] + residual[rows[r]]); x is left as it is.
+// The residual may come in `parts` slices `pstride` elements apart (the K shares of a product):
+// it is then their sum in ascending order, formed first and added to x as one number.
 // The sum, the mean of squares and the scaling are float (reference: tensorline/fused.py:19-32).
 template <typename R, typename O, bool HAS_RES, bool HAS_ROWS>
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const R* __restrict__ res, const float* __restrict__ w,
-                                   O* __restrict__ out, const int32_t* __restrict__ rows, int H, float eps) {
+                                   O* __restrict__ out, const int32_t* __restrict__ rows, int H, float eps, int parts,
+                                   size_t pstride) {
     __shared__ float red[16];
     const int r = blockIdx.x;
     const size_t src = HAS_ROWS ? (size_t)rows[r] : (size_t)r;
@@ -74,7 +77,9 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const R* __restrict__ 
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float v = xr[c];
         if (HAS_RES) {
-            v += tl_to_float(rr[c]);
+            float b = tl_to_float(rr[c]);
+            for (int p = 1; p < parts; ++p) b += tl_to_float(rr[c + p * pstride]);
+            v += b;
             if (!HAS_ROWS) xr[c] = v;
         }
         ss += v * v;
@@ -83,7 +88,11 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const R* __restrict__ 
     const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float v = xr[c];
-        if (HAS_RES && HAS_ROWS) v += tl_to_float(rr[c]);
+        if (HAS_RES && HAS_ROWS) {
+            float b = tl_to_float(rr[c]);
+            for (int p = 1; p < parts; ++p) b += tl_to_float(rr[c + p * pstride]);
+            v += b;
+        }
         orow[c] = tl_from_float<O>(v * rstd * w[c]);
     }
 }
@@ -108,7 +117,8 @@ __device__ __forceinline__ void tl_store4(bf16_t* p, float4 v) {
 template <typename R, typename O, bool HAS_RES, bool HAS_ROWS>
 __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict__ x, const R* __restrict__ res,
                                                                const float* __restrict__ w, O* __restrict__ out,
-                                                               const int32_t* __restrict__ rows, int H, float eps) {
+                                                               const int32_t* __restrict__ rows, int H, float eps,
+                                                               int parts, size_t pstride) {
     __shared__ float red[16];
     const int r = blockIdx.x;
     const size_t src = HAS_ROWS ? (size_t)rows[r] : (size_t)r;
@@ -124,7 +134,14 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict
         if (c4 < n4) {
             float4 a = tl_load4(xr + 4 * c4);
             if (HAS_RES) {
-                const float4 b = tl_load4(rr + 4 * c4);
+                float4 b = tl_load4(rr + 4 * c4);
+                for (int p = 1; p < parts; ++p) {
+                    const float4 e = tl_load4(rr + 4 * c4 + p * pstride);
+                    b.x += e.x;
+                    b.y += e.y;
+                    b.z += e.z;
+                    b.w += e.w;
+                }
                 a.x += b.x;
                 a.y += b.y;
                 a.z += b.z;
@@ -157,41 +174,45 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_vec_kernel(float* __restrict
 
 template <typename R, typename O>
 static void launch_add_rmsnorm(float* x, const R* res, const float* w, O* out, const int32_t* rows, int n_rows,
-                               int H, float eps, hipStream_t stream) {
-    if (H % 4 == 0 && H <= 1024 * 4 * NORM_VPT) {
+                               int H, float eps, int parts, size_t pstride, hipStream_t stream) {
+    if (H % 4 == 0 && H <= 1024 * 4 * NORM_VPT && pstride % 4 == 0) {
         int threads = ((H / 4 + 63) / 64) * 64;
         if (threads > 1024) threads = 1024;
         dim3 grid(n_rows), block(threads);
         if (res && rows)
-            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, true, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, true, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps, parts, pstride);
         else if (res)
-            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, true, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, true, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps, parts, pstride);
         else if (rows)
-            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, false, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, false, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps, parts, pstride);
         else
-            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, false, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<R, O, false, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps, parts, pstride);
         return;
     }
     dim3 grid(n_rows), block(H >= 2048 ? 512 : 256);
     if (res && rows)
-        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, true, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, true, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps, parts, pstride);
     else if (res)
-        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, true, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, true, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps, parts, pstride);
     else if (rows)
-        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, false, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, false, true>), grid, block, 0, stream, x, res, w, out, rows, H, eps, parts, pstride);
     else
-        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, false, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps);
+        hipLaunchKernelGGL((add_rmsnorm_kernel<R, O, false, false>), grid, block, 0, stream, x, res, w, out, rows, H, eps, parts, pstride);
 }
 
-extern "C" int tl_add_rmsnorm(float* x, const void* residual, int res_dtype, const float* w, void* out, int out_dtype,
-                              const int32_t* rows, int n_rows, int H, float eps, hipStream_t stream) {
+extern "C" int tl_add_rmsnorm(float* x, const void* residual, int res_dtype, int res_parts, long long res_part_stride,
+                              const float* w, void* out, int out_dtype, const int32_t* rows, int n_rows, int H,
+                              float eps, hipStream_t stream) {
     TL_CHECK_ARG(n_rows >= 0 && H > 0, "tl_add_rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+    TL_CHECK_ARG(res_parts >= 1 && res_parts <= 64 && (res_parts == 1 || (residual && res_part_stride > 0)),
+                 "tl_add_rmsnorm: bad residual parts %d (stride %lld)", res_parts, res_part_stride);
     TL_CHECK_ARG(eps >= 0.f, "tl_add_rmsnorm: eps must be >= 0");
     if (n_rows == 0) return 0;
     if (!residual) res_dtype = TL_F32;
 #define TL_NORM_CASE(RD, RT, OD, OT)                                                                     \
     if (res_dtype == RD && out_dtype == OD) {                                                            \
-        launch_add_rmsnorm<RT, OT>(x, (const RT*)residual, w, (OT*)out, rows, n_rows, H, eps, stream);  \
+        launch_add_rmsnorm<RT, OT>(x, (const RT*)residual, w, (OT*)out, rows, n_rows, H, eps, res_parts, \
+                                   (size_t)res_part_stride, stream);                                     \
         TL_CHECK_LAUNCH("tl_add_rmsnorm");                                                               \
         return 0;                                                                                        \
     }

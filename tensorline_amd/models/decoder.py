@@ -123,15 +123,20 @@ class DecoderModel:
             if getattr(block, "takes_normed_rows", None) is None:
                 pending = block.forward(x, pending, ctx, caches[i])      # a block that knows no hand-off
                 continue
-            # the norm after this block, if whoever applies it can take it as NormedRows
-            next_norm = None
+            # the norm after this block: as next_norm if whoever applies it can take it as
+            # NormedRows, as pending_norm if it adds a product left in its K shares
+            next_norm = after = None
             if i < last:
                 nxt = self.blocks[self.schedule[i + 1].layer]
+                after = getattr(nxt, "mixer_norm", None)
                 if getattr(nxt, "takes_normed_rows", lambda: False)():
                     next_norm = nxt.mixer_norm
-            elif self.head.shuffled is not None:
-                next_norm = self.final_norm
-            pending = block.forward(x, pending, ctx, caches[i], next_norm=next_norm)
+            else:
+                after = self.final_norm
+                if self.head.shuffled is not None:
+                    next_norm = self.final_norm
+            pending_norm = after if getattr(after, "adds_share_sums", False) else None
+            pending = block.forward(x, pending, ctx, caches[i], next_norm=next_norm, pending_norm=pending_norm)
         if ctx.logit_rows.numel() == 0:
             # the residual stream is complete only after the last add; nothing reads it here
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=x.device)

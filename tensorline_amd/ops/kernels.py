@@ -119,11 +119,18 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = Non
     return out
 
 
-def add_rmsnorm(x: torch.Tensor, residual: torch.Tensor | None, weight: torch.Tensor, eps: float,
+def add_rmsnorm(x: torch.Tensor, residual: "torch.Tensor | ShareSum | None", weight: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: torch.Tensor | None = None,
                 out: torch.Tensor | None = None) -> torch.Tensor:
     """Without ``rows``: ``x += residual`` in place (float32), returns ``RMSNorm(x) * weight``.
-    With ``rows``: returns the norm of ``x[rows] + residual[rows]`` and leaves ``x`` alone."""
+    With ``rows``: returns the norm of ``x[rows] + residual[rows]`` and leaves ``x`` alone.
+    ``residual`` may be a :class:`ShareSum`: its shares are added in order, then to ``x``."""
+    parts, part_stride = 1, 0
+    if isinstance(residual, ShareSum):
+        residual = residual.parts
+        _check(residual.dim() == 3 and residual.is_contiguous(), "add_rmsnorm: shares must be a contiguous [P, T, H] tensor")
+        parts, part_stride = residual.shape[0], residual.shape[1] * residual.shape[2]
+        residual = residual[0]
     _on_gpu(x, residual, weight, rows, out)
     _check(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "add_rmsnorm: x must be contiguous float32 [T, H]")
     T, H = x.shape
@@ -140,7 +147,8 @@ def add_rmsnorm(x: torch.Tensor, residual: torch.Tensor | None, weight: torch.Te
     if out is None:
         out = torch.empty(n, H, dtype=out_dtype, device=x.device)
     _check(out.dtype == out_dtype and out.is_contiguous() and tuple(out.shape) == (n, H), "add_rmsnorm: bad output")
-    _call("tl_add_rmsnorm", _ptr(x), _ptr(residual), res_code, _ptr(weight), _ptr(out), _code(out, "add_rmsnorm out"),
+    _call("tl_add_rmsnorm", _ptr(x), _ptr(residual), res_code, parts, ctypes.c_longlong(part_stride), _ptr(weight),
+          _ptr(out), _code(out, "add_rmsnorm out"),
           _ptr(rows), n, H, ctypes.c_float(eps), _stream())
     return out
 
@@ -194,6 +202,17 @@ class NormSink:
     eps: float
 
 
+@dataclass
+class ShareSum:
+    """A product still in the shares of K it was computed in: ``parts`` [P, M, N] float32 stands for
+    ``parts[0] + parts[1] + ...`` in that order.  The norm kernel adds the shares on its way
+    (:func:`add_rmsnorm`), which saves the pass over memory that adding them first would take."""
+    parts: torch.Tensor
+
+    def sum(self) -> torch.Tensor:
+        return self.parts.sum(0)
+
+
 class _NormArgs(ctypes.Structure):
     _fields_ = [("ss_in", ctypes.c_void_p), ("ss_ld", ctypes.c_int), ("ss_n", ctypes.c_int),
                 ("dim", ctypes.c_float), ("eps", ctypes.c_float),
@@ -238,12 +257,14 @@ def _norm_args(owed: NormedRows | None, sink: NormSink | None, M: int, N: int, d
 
 def linear(a: torch.Tensor | NormedRows, weight: torch.Tensor, bias: torch.Tensor | None = None,
            out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
-           shuffled: torch.Tensor | None = None, sink: NormSink | None = None) -> torch.Tensor | NormedRows:
+           shuffled: torch.Tensor | None = None, sink: NormSink | None = None,
+           keep_shares: bool = False) -> "torch.Tensor | NormedRows | ShareSum":
     """``a @ weight.T + bias``: a [M, K] (rows may be strided), weight [N, K], bias float32 [N].
     ``shuffled``: the copy of ``weight`` made by :func:`shuffle_weight`, which few-row bfloat16
     products stream instead of ``weight``.  ``a`` may be :class:`NormedRows` and ``sink`` a
     :class:`NormSink` (then the result is the next norm's :class:`NormedRows`); both need the few-row
-    kernel (:func:`can_defer_norm` rows, a shuffled copy)."""
+    kernel (:func:`can_defer_norm` rows, a shuffled copy).  ``keep_shares``: the caller takes a
+    :class:`ShareSum` where the product is computed in shares of K (many rows, a long K)."""
     owed = a if isinstance(a, NormedRows) else None
     if owed is not None:
         a = owed.rows
@@ -278,7 +299,7 @@ def linear(a: torch.Tensor | NormedRows, weight: torch.Tensor, bias: torch.Tenso
     if out is None:
         if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and (
                 M > ROWS64_MAX_ROWS or (M > SKINNY_MAX_ROWS and shuffled is None)):
-            return _library_linear(a, weight, bias, out_dtype)
+            return _library_linear(a, weight, bias, out_dtype, keep_shares)
         out = torch.empty(M, N, dtype=out_dtype, device=a.device)
     _check(out.dim() == 2 and tuple(out.shape) == (M, N) and out.stride(1) == 1 and out.dtype == out_dtype,
            "linear: bad output")
@@ -331,7 +352,7 @@ def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled=None) -> 
 _MM_OUT_DTYPE_OK: bool | None = None
 
 
-def _library_linear(a, weight, bias, out_dtype) -> torch.Tensor:
+def _library_linear(a, weight, bias, out_dtype, keep_shares: bool = False):
     """hipBLASLt through torch for many-row bfloat16 products (float32 accumulation inside)."""
     global _MM_OUT_DTYPE_OK
     wt = weight.t()
@@ -346,6 +367,8 @@ def _library_linear(a, weight, bias, out_dtype) -> torch.Tensor:
             kk = K // ks
             parts = torch.bmm(a.view(M, ks, kk).transpose(0, 1), weight.view(N, ks, kk).permute(1, 2, 0),
                               out_dtype=torch.float32)
+            if keep_shares and bias is None:
+                return ShareSum(parts)
             y = parts.sum(0)
             if bias is not None:
                 y.add_(bias)

@@ -46,6 +46,13 @@ class Part:
     # Parts without these never see either object.
     defers_norm = False
 
+    # Optional hand-off of a product's K shares to the norm that adds it to the residual (many-row
+    # bfloat16 steps).  A feed-forward that sets ``keeps_share_sums`` takes a ``keep_shares`` keyword
+    # and may then return :class:`tensorline_amd.ops.kernels.ShareSum` instead of a tensor; a norm
+    # that sets ``adds_share_sums`` takes one as its residual.  The block asks only when both do.
+    keeps_share_sums = False
+    adds_share_sums = False
+
 
 class Linear:
     """``y = x W^T + b`` with W [out, in] as checkpoints store it (reference: tensorline/quant.py:3)."""
@@ -77,9 +84,10 @@ class Linear:
     def tensors_kept(self) -> list[torch.Tensor]:
         return [t for t in (self.weight, self.bias, self.shuffled) if t is not None]
 
-    def __call__(self, x, out_dtype: torch.dtype | None = None, sink=None, with_bias: bool = True):
+    def __call__(self, x, out_dtype: torch.dtype | None = None, sink=None, with_bias: bool = True,
+                 keep_shares: bool = False):
         return kernels.linear(x, self.weight, self.bias if with_bias else None, out_dtype=out_dtype,
-                              shuffled=self.shuffled, sink=sink)
+                              shuffled=self.shuffled, sink=sink, keep_shares=keep_shares)
 
 
 def fuse_linears(name: str, parts: list[Linear]) -> Linear:

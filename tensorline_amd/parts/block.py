@@ -40,11 +40,13 @@ class PreNormBlock:
         """Whether the block before this one may hand over this block's first norm as NormedRows."""
         return _deferrable(self.mixer_norm) is not None and bool(getattr(self.mixer, "defers_norm", False))
 
-    def forward(self, x: torch.Tensor, pending, ctx, cache, next_norm=None):
+    def forward(self, x: torch.Tensor, pending, ctx, cache, next_norm=None, pending_norm=None):
         """Updates the residual stream ``x`` in place; returns the new pending feed-forward output.
-        ``pending`` is a tensor still to be added, None, or the NormedRows of this block's first norm
-        (already added).  ``next_norm``: the norm that will take this block's output, given only
-        when whoever applies it accepts NormedRows; the block may then return them."""
+        ``pending`` is what is still to be added (a tensor, a ShareSum this block's first norm said
+        it adds, or None), or the NormedRows of this block's first norm (already added).
+        ``next_norm``: the norm that will take this block's output, given only when whoever applies
+        it accepts NormedRows; the block may then return them.  ``pending_norm``: the norm that
+        will add what this block returns, if it is one that adds a ShareSum."""
         defer = kernels.can_defer_norm(x.shape[0], self.mixer_norm.dtype)
         h = pending if isinstance(pending, kernels.NormedRows) else self.mixer_norm.forward(x, pending)
         sink = self._sink(defer, x, self.mixer, self.feed_forward_norm, self.feed_forward)
@@ -55,6 +57,8 @@ class PreNormBlock:
         sink = self._sink(defer and next_norm is not None, x, self.feed_forward, next_norm, None)
         if sink is not None:
             return self.feed_forward.forward(h, ctx, sink=sink)
+        if pending_norm is not None and getattr(self.feed_forward, "keeps_share_sums", False):
+            return self.feed_forward.forward(h, ctx, keep_shares=True)
         return self.feed_forward.forward(h, ctx)
 
     @staticmethod

@@ -44,6 +44,8 @@ class SwiGLU(Part):
     def defers_norm(self) -> bool:
         return self.gate_up.shuffled is not None and self.down.shuffled is not None
 
-    def forward(self, h, ctx, sink=None):
+    keeps_share_sums = True
+
+    def forward(self, h, ctx, sink=None, keep_shares: bool = False):
         act = kernels.swiglu_gate_up(h, self.gate_up.weight, self.gate_up.shuffled)
-        return self.down(act, out_dtype=torch.float32, sink=sink)
+        return self.down(act, out_dtype=torch.float32, sink=sink, keep_shares=keep_shares)

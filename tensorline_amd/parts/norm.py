@@ -31,10 +31,11 @@ class RMSNorm(Part):
     def weight_tensors(self):
         return [self.weight]
 
+    adds_share_sums = True
+
     def deferrable(self) -> tuple[torch.Tensor, float]:
         """(weight, eps): all a product needs to carry this norm (see ``Part.defers_norm``)."""
         return self.weight, self.eps
 
-    def forward(self, x: torch.Tensor, residual: torch.Tensor | None = None,
-                rows: torch.Tensor | None = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, residual=None, rows: torch.Tensor | None = None) -> torch.Tensor:
         return kernels.add_rmsnorm(x, residual, self.weight, self.eps, self.dtype, rows=rows)

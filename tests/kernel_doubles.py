@@ -41,7 +41,7 @@ def shuffle_weight(weight):
     return None
 
 
-def linear(a, weight, bias=None, out_dtype=None, out=None, shuffled=None, sink=None):
+def linear(a, weight, bias=None, out_dtype=None, out=None, shuffled=None, sink=None, keep_shares=False):
     assert sink is None, "the stand-ins make no shuffled copies, so no part defers a norm"
     y = a.to(torch.float32) @ weight.to(torch.float32).T
     if bias is not None:

@@ -77,6 +77,45 @@ def test_linear(dtype, M, N, Kd):
     torch.testing.assert_close(got32.double(), a.double() @ w.double().T, **tol(dtype, 1e-5, 1e-5))
 
 
+@pytest.mark.parametrize("H", [896, 193, 3584])
+def test_add_rmsnorm_takes_a_product_in_its_shares(H):
+    """A residual given as the K shares of a product: the shares are added in order, then to x; the
+    result has the bits of adding them first."""
+    torch.manual_seed(H)
+    T, eps = 37, 1e-6
+    w = torch.empty(H, device=DEV).uniform_(0.5, 1.5)
+    for P in (2, 3):
+        x = torch.randn(T, H, device=DEV)
+        x2 = x.clone()
+        parts = torch.randn(P, T, H, device=DEV)
+        got = K().add_rmsnorm(x, K().ShareSum(parts), w, eps, torch.bfloat16)
+        want = K().add_rmsnorm(x2, parts.sum(0), w, eps, torch.bfloat16)
+        torch.testing.assert_close(x, x2, atol=0, rtol=0)
+        torch.testing.assert_close(got, want, atol=0, rtol=0)
+        rows = torch.tensor([5, 0, 36], dtype=torch.int32, device=DEV)
+        got_r = K().add_rmsnorm(x, K().ShareSum(parts), w, eps, torch.float32, rows=rows)
+        want_r = K().add_rmsnorm(x2, parts.sum(0), w, eps, torch.float32, rows=rows)
+        torch.testing.assert_close(got_r, want_r, atol=0, rtol=0)
+
+
+def test_linear_many_rows_keeps_its_shares_on_request():
+    """A many-row product with a long K and few output tiles runs as shares of K: on request they
+    come back unsummed, and their sum is the product."""
+    torch.manual_seed(3)
+    M, N, Kd = 256, 512, 9216
+    a = torch.randn(M, Kd, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(torch.bfloat16)
+    want = a.double() @ w.double().T
+    whole = K().linear(a, w, None, out_dtype=torch.float32)
+    kept = K().linear(a, w, None, out_dtype=torch.float32, keep_shares=True)
+    assert isinstance(kept, K().ShareSum) and kept.parts.shape[1:] == (M, N) and kept.parts.shape[0] > 1
+    torch.testing.assert_close(kept.sum(), whole, atol=0, rtol=0)
+    torch.testing.assert_close(whole.double(), want, atol=2e-3, rtol=2e-3)
+    # a product that is not cut into shares comes back as a tensor either way
+    small = K().linear(a[:, :1024].contiguous(), w[:, :1024].contiguous(), None, out_dtype=torch.float32, keep_shares=True)
+    assert isinstance(small, torch.Tensor)
+
+
 @pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 48, 64])
 @pytest.mark.parametrize("N,Kd", [(1000, 1184), (4608, 3584), (136, 8), (50, 264), (3584, 18944)])
 def test_linear_few_rows_bfloat16(M, N, Kd):
