@@ -7,7 +7,9 @@
 // token with a group of 7 fills 7 of the 16 columns of one tile and a prompt portion fills whole
 // tiles.  The wave walks its share of the keys in blocks of 32 and keeps, per column, the running
 // maximum, the running sum and the output accumulator in float (online softmax; reference:
-// tensorline/paged_attn.py:25-58).  Waves never talk to each other: no LDS, no barriers.
+// tensorline/paged_attn.py:25-58).  In the first kernel (decoded tokens, key splits) waves never
+// talk to each other: no LDS, no barriers.  The second (attn_tile_kernel, steps with prompt
+// portions) shares tiles of keys and values among the eight waves of a work-group through LDS.
 //
 // Matrix-core mapping (v_mfma_f32_16x16x32_bf16, D = A*B, lane l: c = l % 16, g = l / 16):
 //   scores^T [keys x columns] = K [keys x d] * Q^T [d x columns]
