@@ -499,6 +499,7 @@ __device__ __forceinline__ void am_tile_lds(const uint4* kt, const uint4* vt, in
 // then lies in one page and a page id is a shift away.  No key split: a step with prompt portions
 // has columns enough.
 #define AT_KEYS 64
+#define AT_CUS 256                   // compute units of the GPU
 #define AT_NT 1                      // column tiles per wave; 8 / AT_NT waves in a work-group
 // LDS row of key k of a tile (see am_block_lds), and the key of an LDS row
 __device__ __forceinline__ int at_lds_row(int k) {
@@ -590,7 +591,17 @@ __global__ __launch_bounds__(WAVES * 64, 32 / WAVES) void attn_tile_kernel(
     const uint32_t k_stride = (uint32_t)nkv * D * 2;         // bytes from a slot to the next
     const uint32_t v_stride = (uint32_t)nkv * D * bs * 2;    // bytes from a page to the next
     const int kx = at_k_swizzle<UPK>(c), vx = at_v_swizzle(c);
-    const int wg_col0 = (ngroups - 1 - flat) * 128;
+    // Which of its sequence's groups: the one with the most keys first.  The hardware places
+    // work-group i + 256 on the CU of work-group i (256 CUs, two work-groups each), so when the
+    // grid has more than 256 and at most 512 work-groups the groups after the first 256 / nkv are
+    // taken from the light end instead: the heaviest shares its CU with the lightest, and the CUs
+    // finish together instead of the first ones last.
+    int group = ngroups - 1 - flat;
+    {
+        const int total = (int)(gridDim.x * gridDim.y), first = AT_CUS / (int)gridDim.x;
+        if (total > AT_CUS && total <= 2 * AT_CUS && flat >= first) group = flat - first;
+    }
+    const int wg_col0 = group * 128;
     const int col0 = wg_col0 + wave * WCOLS;
     const bool wave_active = col0 < ncols;
 
