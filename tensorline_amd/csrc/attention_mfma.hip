@@ -348,7 +348,7 @@ __device__ __forceinline__ void am_block_lds(const uint4* kt, const uint4* vt, i
         // exceeds it by more than AM_LAZY (in the base-2 domain), so probabilities stay below
         // 2^AM_LAZY and the accumulator is rescaled in few blocks instead of most.  Sums and
         // accumulators stay relative to the same running maximum, so the result is the same.
-        const bool moved = bmax > m_run[j] + AM_LAZY || (m_run[j] == -INFINITY && bmax > -INFINITY);
+        const bool moved = bmax > m_run[j] + AM_LAZY;         // also the first keys: -inf + AM_LAZY is -inf
         const float m_new = moved ? bmax : m_run[j];
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
         float pr[8], psum = 0.f;
@@ -444,7 +444,7 @@ __device__ __forceinline__ void am_tile_lds(const uint4* kt, const uint4* vt, in
                          am_max3(am_max3(sv[7], sv[8], sv[9]), am_max3(sv[10], sv[11], sv[12]), sv[13]), am_max3(sv[14], sv[15], sv[15]));
     bmax = am_column_max(bmax);
     bmax *= scale2;                                          // the scale is positive: the order is the same
-    const bool moved = bmax > m_run + AM_LAZY || (m_run == -INFINITY && bmax > -INFINITY);
+    const bool moved = bmax > m_run + AM_LAZY;               // also the first keys: -inf + AM_LAZY is -inf
     const float m_new = moved ? bmax : m_run;
     const float neg_m = (m_new == -INFINITY) ? 0.f : -m_new;
     float pr[16];
