@@ -129,6 +129,7 @@ def bench_decode(llm, batch: int, context: int, steps: int, warmup: int, seed: i
 def bench_prefill(llm, tokens: int, reps: int, seed: int) -> dict:
     """One prompt of ``tokens`` tokens in one step, logits for its last position."""
     from tensorline_amd.engine.batch import StepEntry
+    from tensorline_amd.ops import kernels
     cfg = llm.model_config
     cache, runner = llm.cache, llm.engine.runner
     prompt = random_prompts(1, tokens, cfg.vocab_size, seed)[0]
@@ -140,7 +141,7 @@ def bench_prefill(llm, tokens: int, reps: int, seed: int) -> dict:
         sync()
         t0 = time.perf_counter()
         logits = runner.step([StepEntry(rid, prompt, 0, [tokens - 1])])
-        logits.argmax(-1).tolist()
+        kernels.argmax(logits).tolist()                                # the engine's greedy pick, as in a decode step
         sync()
         times.append(time.perf_counter() - t0)
         cache.release(rid)
