@@ -75,6 +75,40 @@ def test_first_tokens_and_long_decode(setup, dtype):
     _compare(got, {k: v for k, v in want.items() if k[0] == rid}, one, LIMIT[dtype])
 
 
+def test_wide_feed_forward_whose_product_comes_in_shares(tmp_path, monkeypatch):
+    """A feed-forward so wide (8,192) that many-row steps compute the down projection in shares of
+    K, which the next norm adds: whole prompts and portions against the plain implementation, and a
+    step of few rows (no shares) beside them."""
+    from tensorline_amd.config import Qwen2Config
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.replay import TraceSession
+    from tensorline_amd.weights import write_random_model
+    cfg_dict = dict(architectures=["Qwen2ForCausalLM"], vocab_size=300, hidden_size=96, intermediate_size=8192,
+                    num_hidden_layers=2, num_attention_heads=3, num_key_value_heads=1, head_dim=32,
+                    rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=512)
+    d = write_random_model(Qwen2Config.from_dict(cfg_dict), str(tmp_path / "wide"), seed=2)
+    w, cfg = plain.load_folder(d)
+    import random
+    rng = random.Random(1)
+    reqs = {f"r{i}": [rng.randrange(300) for _ in range(n)] for i, n in enumerate([150, 9, 260])}
+    want = helpers.plain_logits(w, cfg, reqs)
+    model, _ = load_model(d, "bfloat16", "cuda:0")
+    from tensorline_amd.ops import kernels
+    made = []
+
+    class CountedShareSum(kernels.ShareSum):
+        def __init__(self, parts):
+            super().__init__(parts)
+            made.append(parts.shape[0])
+    monkeypatch.setattr(kernels, "ShareSum", CountedShareSum)
+    for steps in (helpers.steps_whole(reqs), helpers.steps_portions(reqs, sizes=(100, 70, 3, 90))):
+        session = TraceSession(model, helpers.max_live_tokens(steps), page_size=16)
+        got = helpers.collect_logits(session.step, steps)
+        _compare(got, want, reqs, LIMIT["bfloat16"])
+        assert session.cache.all_free()
+    assert made and min(made) > 1, "no step computed the down projection in shares"
+
+
 def test_trace_run_program(setup, tmp_path):
     """bin/trace_run as a user calls it: JSON lines in, <step>.f32 files and 'done' lines out."""
     name, d, reqs, want = setup
