@@ -44,7 +44,8 @@ template <int P, bool PAIR>
 __device__ __forceinline__ void r64_issue(const bf16_t* const (&xp)[P], const uint4* w1, const uint4* w2, int step,
                                           int xunit, int K, int last_c, uint4 (&xo)[P], uint4 (&wo)[4],
                                           uint4 (&uo)[PAIR ? 4 : 1]) {
-    const int kbase = (step * R64_SC + xunit * 8 < K) ? step * R64_SC : 0;
+    // past K: the row's first unit, which lies inside the row whatever K is
+    const int kbase = (step * R64_SC + xunit * 8 < K) ? step * R64_SC + xunit * 8 : 0;
 #pragma unroll
     for (int i = 0; i < P; ++i) xo[i] = *reinterpret_cast<const uint4*>(xp[i] + kbase);
 #pragma unroll
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(THREADS) void gemm_rows64_kernel(
         const int idx = tid + nthreads * i;
         xmine[i] = idx < R64_PIECES;
         const int row = xmine[i] ? idx >> 4 : 0, unit = idx & 15;
-        xp[i] = A + (size_t)(row < M ? row : 0) * lda + unit * 8;
+        xp[i] = A + (size_t)(row < M ? row : 0) * lda;       // the row's start: the unit (this thread's xunit) is part of the k offset
         xslot[i] = ((row >> 4) * R64_UNITS + unit) * R64_ROWPAD + (row & 15);
     }
     const int xunit = tid & 15;

@@ -144,13 +144,13 @@ __global__ __launch_bounds__(MODE == MODE_SWIGLU ? 256 : 512) void gemm_skinny_k
 #pragma unroll
     for (int i = 0; i < MT * 4; ++i) {
         const int row = xrow0 + 4 * i;
-        xp[i] = A + (size_t)(row < M ? row : 0) * lda + xunit * 8;
+        xp[i] = A + (size_t)(row < M ? row : 0) * lda;       // the row's start: the unit is part of the k offset
     }
     const int last_c = K32 - 1;
     {
         const int sc = (s0 < s1) ? s0 : 0;
         const int kx = sc * SK_SC + xunit * 8;
-        const int kxc = (kx < K) ? sc * SK_SC : 0;
+        const int kxc = (kx < K) ? kx : 0;               // past K: the row's first unit, inside the row whatever K is
 #pragma unroll
         for (int i = 0; i < MT * 4; ++i) xr[i] = *reinterpret_cast<const uint4*>(xp[i] + kxc);
         if (kx >= K) {
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(MODE == MODE_SWIGLU ? 256 : 512) void gemm_skinny_k
         // request the next step (clamped to the last one when there is none)
         const int sn = (sc + 1 < s1) ? sc + 1 : sc;
         const int kxn = sn * SK_SC + xunit * 8;
-        const int kxnc = (kxn < K) ? sn * SK_SC : 0;
+        const int kxnc = (kxn < K) ? kxn : 0;
 #pragma unroll
         for (int i = 0; i < MT * 4; ++i) xr[i] = *reinterpret_cast<const uint4*>(xp[i] + kxnc);
 #pragma unroll
