@@ -148,12 +148,14 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, int nq, int nkv, int bs, int bs_shift, int window, float scale, int nsplit,
-    int split_blocks) {
+    int split_blocks, const int32_t* __restrict__ seq_list, int skip_single) {
     constexpr int D = DC * 32;
     constexpr int DB = D / 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = lane & 15, g = lane >> 4;
-    const int s = blockIdx.x, kvh = blockIdx.y;
+    // With a list the grid runs over the listed sequences only (one-token sequences of a step that
+    // also holds prompt portions), and their partial results lie in the workspace by list place.
+    const int s = seq_list ? seq_list[blockIdx.x] : (int)blockIdx.x, kvh = blockIdx.y;
     const int widx = blockIdx.z * (blockDim.x >> 6) + wave;    // one to four waves per work-group
     const int tg = widx / nsplit, sp = widx - tg * nsplit;
     const int G = nq / nkv;
@@ -164,6 +166,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
     const int ncols = n * G;
     const int col0 = tg * NT * 16;
     if (col0 >= ncols) return;
+    if (seq_list ? n != 1 : (skip_single && n == 1)) return;   // another launch of the step owns it
+    const int ws_shift = seq_list ? (int)blockIdx.x - r0 : 0;
     const int32_t* table = tables + (size_t)s * NB;
 
     // ---- this lane's column of each tile ----
@@ -285,7 +289,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
                 *reinterpret_cast<uint2*>(op + db * 16) = w;
             }
         } else {
-            const size_t part = ((size_t)row_col[j] * nq + head_col[j]) * nsplit + sp;
+            const size_t part = ((size_t)(row_col[j] + ws_shift) * nq + head_col[j]) * nsplit + sp;
             float* wp = ws_o + part * D + 4 * g;
 #pragma unroll
             for (int db = 0; db < DB; ++db)
@@ -534,7 +538,7 @@ __global__ __launch_bounds__(WAVES * 64, 32 / WAVES) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int S, int nq, int nkv, int bs,
-    int bs_shift, int window, float scale) {
+    int bs_shift, int window, float scale, int skip_single) {
     constexpr int THREADS = WAVES * 64;
     constexpr int WCOLS = NT * 16;                       // columns of a wave; WAVES * WCOLS = 128 per work-group
     constexpr int D = DC * 32;
@@ -559,7 +563,8 @@ __global__ __launch_bounds__(WAVES * 64, 32 / WAVES) void attn_tile_kernel(
     __syncthreads();
     int s = 0, flat = blockIdx.y, ngroups = 0;
     for (; s < S; ++s) {
-        ngroups = ((qst[s + 1] - qst[s]) * G + 127) / 128;
+        const int nn = qst[s + 1] - qst[s];
+        ngroups = (skip_single && nn == 1) ? 0 : (nn * G + 127) / 128;   // one-token sequences: another launch's
         if (flat < ngroups) break;
         flat -= ngroups;
     }
@@ -751,16 +756,18 @@ static size_t at_lds_bytes(int DC, int pages, int S) {
 template <int AM_MERGE_THREADS>
 __global__ __launch_bounds__(AM_MERGE_THREADS) void attn_merge_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml, const int32_t* __restrict__ pos,
-    bf16_t* __restrict__ out, int out_stride, int nq, int D, int nsplit, int split_blocks, int window) {
+    bf16_t* __restrict__ out, int out_stride, int nq, int D, int nsplit, int split_blocks, int window,
+    const int32_t* __restrict__ seq_list, const int32_t* __restrict__ q_start) {
     __shared__ float wgt[AM_MAX_SPLITS];
     __shared__ float red_m[AM_MERGE_THREADS / 64], red_l[AM_MERGE_THREADS / 64];
     __shared__ float4 part[AM_MERGE_THREADS];
-    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int wrow = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int t = seq_list ? q_start[seq_list[wrow]] : wrow;   // listed one-token sequences: their row of the step
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int s_lo = (lo >> 5) / split_blocks, s_hi = (p >> 5) / split_blocks;
     const int ns = s_hi - s_lo + 1;
-    const size_t base = ((size_t)t * nq + h) * nsplit + s_lo;
+    const size_t base = ((size_t)wrow * nq + h) * nsplit + s_lo;
     const int D4 = D >> 2, SG = AM_MERGE_THREADS / D4;      // D is 32, 64 or 128
     const int d4 = tid % D4, sg = tid / D4;
     const float4* acc4 = reinterpret_cast<const float4*>(ws_o) + base * D4 + d4;
@@ -839,18 +846,19 @@ template <int DC>
 static void launch_attn(int NT, dim3 grid, int wg_waves, hipStream_t stream, const bf16_t* q, int q_stride, const bf16_t* kc,
                         const bf16_t* vc, const int32_t* tables, int NB, const int32_t* q_start,
                         const int32_t* ctx_start, bf16_t* out, int out_stride, float* ws_o, float* ws_ml, int nq, int nkv,
-                        int bs, int window, float scale, int nsplit, int split_blocks) {
+                        int bs, int window, float scale, int nsplit, int split_blocks, const int32_t* seq_list,
+                        int skip_single) {
     int bs_shift = -1;                               // pages of a power of two of tokens: a shift finds the page
     if ((bs & (bs - 1)) == 0)
         for (bs_shift = 0; (1 << bs_shift) < bs;) ++bs_shift;
     if (NT == 1)
         hipLaunchKernelGGL((attn_mfma_kernel<DC, 1>), grid, dim3(64 * wg_waves), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
                            ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
-                           split_blocks);
+                           split_blocks, seq_list, skip_single);
     else
         hipLaunchKernelGGL((attn_mfma_kernel<DC, 2>), grid, dim3(64 * wg_waves), 0, stream, q, q_stride, kc, vc, tables, NB, q_start,
                            ctx_start, out, out_stride, ws_o, ws_ml, nq, nkv, bs, bs_shift, window, scale, nsplit,
-                           split_blocks);
+                           split_blocks, seq_list, skip_single);
 }
 
 // q: bfloat16 [T, >= nq*d] (row stride q_stride); k_cache [pages, page, nkv, d]; v_cache
@@ -861,12 +869,17 @@ static void launch_attn(int NT, dim3 grid, int wg_waves, hipStream_t stream, con
 // (the tokens' positions), ws_o holds T*nq*nsplit*d floats and ws_ml T*nq*nsplit*2.  shared != 0
 // runs unsplit steps with prompt portions on the kernel that shares keys and values through LDS
 // (when the page size and the table length allow it); shared == 0 keeps them on independent waves.
+// A step that holds prompt portions and one-token sequences with long contexts may be run as two
+// calls: one with seq_list (int32 [n_list], the indices of one-token sequences; only they are
+// computed, with split keys, and the workspace then holds n_list rows instead of T), and one
+// with skip_single != 0, which leaves sequences of one token out.
 // total_groups128: the sum over the sequences of ceil(n_s * G / 128), that kernel's grid.
 extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                  const int32_t* tables, int NB, const int32_t* q_start, const int32_t* ctx_start,
                                  const int32_t* pos, void* out, int out_stride, float* ws_o, float* ws_ml, int T, int S,
                                  int nq, int nkv, int d, int bs, int window, float scale, int NT, int max_tile_groups,
-                                 int nsplit, int split_blocks, int shared, int total_groups128, hipStream_t stream) {
+                                 int nsplit, int split_blocks, int shared, int total_groups128,
+                                 const int32_t* seq_list, int n_list, int skip_single, hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && NB > 0, "tl_attention_mfma: bad sizes T=%d S=%d nq=%d nkv=%d NB=%d", T, S, nq, nkv, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_mfma: %d query heads are not a multiple of %d key/value heads", nq, nkv);
     TL_CHECK_ARG(d == 32 || d == 64 || d == 128, "tl_attention_mfma: head size %d is not one of 32, 64, 128", d);
@@ -884,16 +897,20 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
                  "tl_attention_mfma: the split workspace must be 16-byte aligned");
     TL_CHECK_ARG(nkv <= 65535, "tl_attention_mfma: too many key/value heads");
     TL_CHECK_ARG(scale > 0.f, "tl_attention_mfma: the score scale %g must be positive", (double)scale);
-    if (T == 0 || S == 0) return 0;
+    TL_CHECK_ARG(!seq_list || (n_list >= 0 && n_list <= S && !skip_single),
+                 "tl_attention_mfma: a list of %d sequences does not fit %d sequences, or it comes with skip_single", n_list, S);
+    if (T == 0 || S == 0 || (seq_list && n_list == 0)) return 0;
+    const int S_run = seq_list ? n_list : S;               // sequences the grid runs over
     const long waves = (long)max_tile_groups * nsplit;
     // The waves are independent: four to a work-group, fewer when that would leave compute units without one.
     int wg_waves = 4;
-    while (wg_waves > 1 && (long)S * nkv * ((waves + wg_waves - 1) / wg_waves) < 256) wg_waves >>= 1;
+    while (wg_waves > 1 && (long)S_run * nkv * ((waves + wg_waves - 1) / wg_waves) < 256) wg_waves >>= 1;
     TL_CHECK_ARG((waves + wg_waves - 1) / wg_waves <= 65535, "tl_attention_mfma: too many tile groups x splits (%ld)", waves);
-    dim3 grid(S, nkv, (unsigned)((waves + wg_waves - 1) / wg_waves));
+    dim3 grid(S_run, nkv, (unsigned)((waves + wg_waves - 1) / wg_waves));
     const bf16_t *qq = (const bf16_t*)q, *kk = (const bf16_t*)k_cache, *vv = (const bf16_t*)v_cache;
     const bool pow2 = (bs & (bs - 1)) == 0;
-    if (NT == 2 && nsplit == 1 && shared && pow2 && total_groups128 > 0 && at_lds_bytes(d / 32, NB, S) <= 160 * 1024) {
+    if (NT == 2 && nsplit == 1 && shared && pow2 && !seq_list && total_groups128 > 0 &&
+        at_lds_bytes(d / 32, NB, S) <= 160 * 1024) {
         // 128 columns per work-group, keys and values shared through LDS
         int bs_shift = 0;
         while ((1 << bs_shift) < bs) ++bs_shift;
@@ -903,7 +920,7 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
 #define TL_TILE_CASE(DCV)                                                                                             \
     hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT>), sgrid, dim3(64 * 8 / AT_NT), lds, stream, qq,        \
                        q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, S, nq, nkv, bs,     \
-                       bs_shift, window, scale)
+                       bs_shift, window, scale, skip_single)
         if (d == 32) TL_TILE_CASE(1);
         else if (d == 64) TL_TILE_CASE(2);
         else TL_TILE_CASE(4);
@@ -913,21 +930,22 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     }
     if (d == 32)
         launch_attn<1>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
     else if (d == 64)
         launch_attn<2>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
     else
         launch_attn<4>(NT, grid, wg_waves, stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride,
-                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks);
+                       ws_o, ws_ml, nq, nkv, bs, window, scale, nsplit, split_blocks, seq_list, skip_single);
     TL_CHECK_LAUNCH("tl_attention_mfma");
     if (nsplit > 1) {
+        const int merge_rows = seq_list ? n_list : T;
         if (nsplit > 32)
-            hipLaunchKernelGGL(attn_merge_kernel<256>, dim3(T, nq), dim3(256), 0, stream, ws_o, ws_ml, pos,
-                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window);
+            hipLaunchKernelGGL(attn_merge_kernel<256>, dim3(merge_rows, nq), dim3(256), 0, stream, ws_o, ws_ml, pos,
+                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window, seq_list, q_start);
         else
-            hipLaunchKernelGGL(attn_merge_kernel<128>, dim3(T, nq), dim3(128), 0, stream, ws_o, ws_ml, pos,
-                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window);
+            hipLaunchKernelGGL(attn_merge_kernel<128>, dim3(merge_rows, nq), dim3(128), 0, stream, ws_o, ws_ml, pos,
+                               (bf16_t*)out, out_stride, nq, d, nsplit, split_blocks, window, seq_list, q_start);
         TL_CHECK_LAUNCH("tl_attention_mfma merge");
     }
     return 0;

@@ -34,6 +34,9 @@ class AttentionPlan:
     num_seqs: int = 0
     q_lens: list[int] = field(default_factory=list)
     starts: list[int] = field(default_factory=list)
+    # In a step that mixes prompt portions with one-token sequences: the indices of the latter
+    # (also on the device, ``StepContext.single_seqs``), so that they can be given to a kernel of their own.
+    singles: list[int] = field(default_factory=list)
 
 
 @dataclass
@@ -59,6 +62,7 @@ class StepContext:
     state_slots: torch.Tensor         # int32 [S]
     logit_rows: torch.Tensor          # int32 [R]
     attention_plan: AttentionPlan
+    single_seqs: torch.Tensor | None = None   # int32 [len(attention_plan.singles)], if there are any
     # host mirrors, for parts that loop over sequences on the host
     host_q_start: list[int] = field(default_factory=list)
     host_ctx_start: list[int] = field(default_factory=list)
@@ -182,6 +186,9 @@ def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[
     pieces: list[tuple[str, np.ndarray]] = [
         ("ids", ids), ("pos", pos), ("seq_of_token", seq_of), ("q_start", q_start), ("ctx_start", ctx_start),
         ("state_slots", slots_state), ("logit_rows", np.asarray(rows, np.int32))]
+    decode_only = all(n == 1 for n in q_lens)
+    singles = [] if decode_only else [s for s, n in enumerate(q_lens) if n == 1] + list(range(S, S_pad))
+    pieces.append(("single_seqs", np.asarray(singles, np.int32)))
     for g in range(num_groups):
         pieces.append((f"slots{g}", g_slots[g]))
         pieces.append((f"tables{g}", g_tables[g].reshape(-1)))
@@ -193,7 +200,7 @@ def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[
     starts = [e.start for e in entries]
     plan = AttentionPlan(
         max_context=max(st + n for st, n in zip(starts, q_lens)), max_query_len=max(q_lens),
-        decode_only=all(n == 1 for n in q_lens), num_seqs=S_pad, q_lens=q_lens, starts=starts)
+        decode_only=decode_only, num_seqs=S_pad, q_lens=q_lens, starts=starts, singles=singles)
     return PackedBatch(data.astype(np.int32, copy=False), T, S_pad, len(rows), offsets, group_nb, plan,
                        [int(v) for v in q_start], [int(v) for v in ctx_start], [int(v) for v in slots_state],
                        logits_for_all_rows=rows == list(range(T)))

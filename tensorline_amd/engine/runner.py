@@ -60,7 +60,8 @@ class ModelRunner:
             seq_of_token=view("seq_of_token"), q_start=view("q_start"), ctx_start=view("ctx_start"),
             state_slots=view("state_slots"), logit_rows=view("logit_rows"), attention_plan=packed.plan,
             host_q_start=packed.host_q_start, host_ctx_start=packed.host_ctx_start,
-            host_state_slots=packed.host_state_slots, logits_for_all_rows=packed.logits_for_all_rows)
+            host_state_slots=packed.host_state_slots, logits_for_all_rows=packed.logits_for_all_rows,
+            single_seqs=view("single_seqs") if packed.plan.singles else None)
         cache = self.cache
         g_slots = [view(f"slots{g}") for g in range(len(cache.groups))]
         g_tables = [view(f"tables{g}").view(packed.S, packed.group_nb[g]) for g in range(len(cache.groups))]

@@ -557,11 +557,42 @@ def rope_store(qkv: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor | No
           k_cache.shape[1] if write else 0, _ptr(bias), _stream())
 
 
+def _singles_get_own_launch(plan, singles: list[int], num_heads: int, num_kv_heads: int, head_dim: int,
+                            window: int) -> bool:
+    """Whether the one-token sequences of a step with prompt portions are worth a launch of their
+    own.  Beside the portions each of them is walked by one work-group from its first key to its
+    last, about 14 ns a key at a head size of 128 (and never faster than 1.5 times what their
+    bytes take at the streaming rate); that time hides behind the portions' own, about 600 TFLOP/s
+    of their scores and sums.  Alone they run split at the rate a decode step reads its cache,
+    after about 9 us for the two launches, and the portions follow.  (Measured at 28 query and
+    4 key/value heads of 128; only the choice of launches depends on it, not a result.)"""
+    ctxs = [plan.starts[s] + 1 if s < len(plan.starts) else 1 for s in singles]
+    if window > 0:
+        ctxs = [min(c, window) for c in ctxs]
+    stream_us = sum(ctxs) * 4 * num_kv_heads * head_dim / 4.5e6
+    walk_us = max(0.014 * max(ctxs) * max(head_dim, 64) / 128, 1.5 * stream_us)
+    portions_us = sum(n * (st + (n + 1) / 2) for n, st in zip(plan.q_lens, plan.starts) if n > 1) \
+        * num_heads * head_dim * 4 / 6e8
+    return walk_us > portions_us + 9 + stream_us + 5
+
+
+def _key_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> tuple[int, int]:
+    """(keys per split, number of splits) for ``num_seqs`` one-token sequences; (0, 1): no split."""
+    base = (1 << max(num_seqs - 1, 0).bit_length()) * num_kv_heads
+    split_len = 64 if base <= 8 else 128 if base <= 32 else 256 if base <= 128 else 512 if base <= 512 else 0
+    if not split_len:
+        return 0, 1
+    while -(-max_context // split_len) > MAX_KEY_SPLITS:    # very long contexts: longer splits
+        split_len *= 2
+    return split_len, max(1, -(-max_context // split_len))
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, tables: torch.Tensor,
                     seq_of_token: torch.Tensor, pos: torch.Tensor, num_heads: int, num_kv_heads: int,
                     head_dim: int, scale: float, window: int = 0, out: torch.Tensor | None = None,
                     q_start: torch.Tensor | None = None, ctx_start: torch.Tensor | None = None, plan=None,
-                    path: str | None = None, split_keys: int | None = None) -> torch.Tensor:
+                    path: str | None = None, split_keys: int | None = None,
+                    single_seqs: torch.Tensor | None = None, route_singles: bool | None = None) -> torch.Tensor:
     """Causal attention of each token over the cached keys of its sequence.
 
     ``q``: [T, >= nq*d] with the query heads in the first nq*d columns (row stride free);
@@ -573,7 +604,14 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     and the host-side ``plan`` (lengths of the step's sequences).  Everything else runs the
     any-shape kernel.  ``path`` forces one: "generic", "mfma" (prompt portions on the kernel that
     shares key tiles through LDS where the page size allows) or "mfma-direct" (independent waves);
-    ``split_keys`` forces the number of keys per split (0: no split)."""
+    ``split_keys`` forces the number of keys per split (0: no split).
+
+    A step with prompt portions does not split keys: its one-token sequences would each be walked
+    by one work-group from the first key to the last.  With ``single_seqs`` (int32, the indices
+    ``plan.singles`` on the device) they are computed by a launch of their own where that is
+    estimated to be faster (``_singles_get_own_launch``), split like a decode step of that many
+    sequences, and the launch for the portions leaves them out.  ``route_singles`` forces that
+    on or off."""
     _on_gpu(q, k_cache, v_cache, tables, seq_of_token, pos, out, q_start, ctx_start)
     T = q.shape[0]
     _check(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= num_heads * head_dim, "paged_attention: bad query layout")
@@ -597,11 +635,29 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _i32(q_start, "q_start", S + 1)
         _i32(ctx_start, "ctx_start", S)
         G = num_heads // num_kv_heads
+        skip_single = 0
+        singles = plan.singles if single_seqs is not None and not plan.decode_only and split_keys is None else []
+        if singles and route_singles is not False:
+            _i32(single_seqs, "single_seqs", len(singles))
+            ctx1 = max([plan.starts[s] + 1 for s in singles if s < len(plan.starts)] + [1])
+            split_len, nsplit = _key_splits(len(singles), num_kv_heads, ctx1)
+            if route_singles or (route_singles is None and nsplit > 1 and _singles_get_own_launch(
+                    plan, singles, num_heads, num_kv_heads, head_dim, int(window))):
+                nt1 = 1 if G <= 16 else 2
+                ws = torch.empty(len(singles) * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
+                n_o = len(singles) * num_heads * nsplit * head_dim
+                _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
+                      _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws[:n_o]), _ptr(ws[n_o:]), T, S,
+                      num_heads, num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt1,
+                      -(-G // (16 * nt1)), nsplit, max(split_len // 32, 1), 0, 0, _ptr(single_seqs), len(singles), 0,
+                      _stream())
+                skip_single = 1
+        q_lens = [n for n in plan.q_lens if n > 1] if skip_single else plan.q_lens
         nt = 1 if plan.max_query_len * G <= 16 else 2
-        groups = [-(-n * G // (16 * nt)) for n in plan.q_lens]
-        pads = max(0, S - len(groups))                     # padding sequences bring one token each
+        groups = [-(-n * G // (16 * nt)) for n in q_lens]
+        pads = 0 if skip_single else max(0, S - len(groups))    # padding sequences bring one token each
         max_groups = max(groups + [1])
-        total128 = sum(-(-n * G // 128) for n in plan.q_lens) + pads
+        total128 = sum(-(-n * G // 128) for n in q_lens) + pads
         # Splits are fixed runs of keys aligned to absolute positions, so the same keys are summed
         # together whatever the context length or the launch shape.  Pure decode steps split by the
         # batch size rounded up to a power of two (what a graph bucket pads to); steps with prompt
@@ -610,8 +666,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if split_keys is not None:
             split_len = int(split_keys)
         elif plan.decode_only:
-            base = (1 << max(S - 1, 0).bit_length()) * num_kv_heads
-            split_len = 64 if base <= 8 else 128 if base <= 32 else 256 if base <= 128 else 512 if base <= 512 else 0
+            split_len, _ = _key_splits(S, num_kv_heads, plan.max_context)
         nsplit, split_blocks = 1, 1
         if split_len:
             _check(split_len % 32 == 0, "paged_attention: a split is a multiple of 32 keys")
@@ -626,7 +681,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
               _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,
               num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,
-              0 if path == "mfma-direct" else 1, total128, _stream())
+              0 if path == "mfma-direct" else 1, total128, _ptr(None), 0, skip_single, _stream())
         return out
     _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
           _ptr(seq_of_token), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, num_heads,

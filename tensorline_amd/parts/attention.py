@@ -97,5 +97,5 @@ class PagedAttention(Part):
         o = kernels.paged_attention(qkv, cache.k, cache.v, cache.tables, ctx.seq_of_token, ctx.pos,
                                     self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
                                     window=self.window, q_start=ctx.q_start, ctx_start=ctx.ctx_start,
-                                    plan=ctx.attention_plan)
+                                    plan=ctx.attention_plan, single_seqs=ctx.single_seqs)
         return self.o_proj(o, out_dtype=torch.float32, sink=sink)

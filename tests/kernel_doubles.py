@@ -75,7 +75,8 @@ def rope_store(qkv, pos, inv_freq, num_heads, num_kv_heads, head_dim, k_cache, v
 
 
 def paged_attention(q, k_cache, v_cache, tables, seq_of_token, pos, num_heads, num_kv_heads, head_dim, scale,
-                    window=0, out=None, q_start=None, ctx_start=None, plan=None, path=None, split_keys=None):
+                    window=0, out=None, q_start=None, ctx_start=None, plan=None, path=None, split_keys=None,
+                    single_seqs=None, route_singles=None):
     T, d, bs = q.shape[0], head_dim, k_cache.shape[1]
     g = num_heads // num_kv_heads
     o = torch.empty(T, num_heads * d, dtype=q.dtype)

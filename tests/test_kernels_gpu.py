@@ -342,7 +342,8 @@ def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
     torch.testing.assert_close(got, want2, atol=2e-2, rtol=2e-2)
 
 
-def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False, path=None, split_keys=None):
+def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False, path=None, split_keys=None,
+                    route_singles=None):
     """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries."""
     torch.manual_seed(seed)
     S = len(lens)
@@ -373,11 +374,15 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
         qs.append(qs[-1] + ql)
     plan = AttentionPlan(max_context=max(lens), max_query_len=max(q_lens), decode_only=max(q_lens) == 1,
                          num_seqs=S, q_lens=list(q_lens), starts=[n - ql for n, ql in zip(lens, q_lens)])
+    single_seqs = None
+    if not plan.decode_only and 1 in q_lens:
+        plan.singles = [s for s, ql in enumerate(q_lens) if ql == 1]
+        single_seqs = torch.tensor(plan.singles, dtype=torch.int32, device=DEV)
     out = K().paged_attention(q, kc, vc, tables, torch.tensor(seq_of, dtype=torch.int32, device=DEV),
                               torch.tensor(pos, dtype=torch.int32, device=DEV), nq, nkv, d, d ** -0.5, window=window,
                               q_start=torch.tensor(qs, dtype=torch.int32, device=DEV),
                               ctx_start=torch.tensor(plan.starts, dtype=torch.int32, device=DEV), plan=plan,
-                              path=path, split_keys=split_keys)
+                              path=path, split_keys=split_keys, single_seqs=single_seqs, route_singles=route_singles)
     kf, vf = kc.double().cpu().view(-1, nkv, d), vc.double().cpu().permute(0, 3, 1, 2).reshape(-1, nkv, d)
     want = torch.empty(T, nq, d, dtype=torch.float64)
     tcpu = tables.cpu().long()
@@ -450,6 +455,32 @@ def test_attention_matrix_core_kernel(path, heads, d):
             got, want = _attention_case(dtype, heads[0], heads[1], d, 16, [50, 7, 130, 700], [20, 7, 1, 33],
                                         window=window, seed=9, path=path, split_keys=split_keys)
             torch.testing.assert_close(got, want, atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("heads", [(14, 2), (4, 4), (28, 4), (40, 2)])
+@pytest.mark.parametrize("d,bs", [(32, 16), (64, 24), (128, 16), (128, 8)])
+def test_attention_one_token_sequences_beside_prompt_portions(heads, d, bs):
+    """In a step with prompt portions the one-token sequences may be computed by a launch of their
+    own with split keys (they are, by default, when their contexts are long beside the portions): first,
+    last and between portions, contexts of one key and of thousands, a dominating far key, a
+    window, pages of no power of two (where the portions run on independent waves)."""
+    dtype = torch.bfloat16
+    lens = [5000, 40, 1, 1400, 700, 31, 2, 1025]
+    q_lens = [1, 40, 1, 1, 300, 1, 2, 1]
+    for window in (0, 100):
+        outs = []
+        for route in (True, False, None):
+            got, want = _attention_case(dtype, heads[0], heads[1], d, bs, lens, q_lens, window=window, seed=11,
+                                        spike=window == 0, route_singles=route)
+            torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+            outs.append(got)
+        if window == 0:
+            assert torch.equal(outs[0], outs[2])              # 5,000 keys: routed when left to choose
+        portion_rows = [r for r in range(sum(q_lens)) if r not in (0, 41, 42, 343, sum(q_lens) - 1)]
+        assert torch.equal(outs[0][portion_rows], outs[1][portion_rows])
+    short = _attention_case(dtype, heads[0], heads[1], d, bs, [500, 40, 9], [1, 40, 1], seed=12, route_singles=None)
+    unrouted = _attention_case(dtype, heads[0], heads[1], d, bs, [500, 40, 9], [1, 40, 1], seed=12, route_singles=False)
+    assert torch.equal(short[0], unrouted[0])                 # short contexts stay with the portions
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

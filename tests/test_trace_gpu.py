@@ -75,6 +75,33 @@ def test_first_tokens_and_long_decode(setup, dtype):
     _compare(got, {k: v for k, v in want.items() if k[0] == rid}, one, LIMIT[dtype])
 
 
+def test_mixed_steps_with_one_token_sequences_on_a_launch_of_their_own(setup, monkeypatch):
+    """Steps that hold prompt portions beside decoded tokens give the latter's attention to a
+    separate launch with split keys once their contexts are long; here whenever keys are split, so
+    that the tiny configurations take that way, with few pages, against the plain implementation."""
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.replay import TraceSession
+    from tensorline_amd.ops import kernels
+    name, d, reqs, want = setup
+    monkeypatch.setattr(kernels, "_singles_get_own_launch", lambda *a: True)
+    routed = []
+    call = kernels._call
+
+    def counting(fn, *args):
+        if fn == "tl_attention_mfma" and args[-4].value:       # the list of one-token sequences
+            routed.append(args[-3])
+        return call(fn, *args)
+    monkeypatch.setattr(kernels, "_call", counting)
+    steps = helpers.steps_mixed(reqs)
+    model, cfg = load_model(d, "bfloat16", "cuda:0")
+    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=helpers.PAGE[name])
+    got = helpers.collect_logits(session.step, steps)
+    _compare(got, want, reqs, LIMIT["bfloat16"])
+    assert session.cache.all_free()
+    if cfg.head_dim in (32, 64, 128):                 # other head sizes run the any-shape kernel
+        assert routed and max(routed) >= 1, "no step gave its one-token sequences a launch of their own"
+
+
 def test_wide_feed_forward_whose_product_comes_in_shares(tmp_path, monkeypatch):
     """A feed-forward so wide (8,192) that many-row steps compute the down projection in shares of
     K, which the next norm adds: whole prompts and portions against the plain implementation, and a
