@@ -505,10 +505,8 @@ __device__ __forceinline__ void am_tile_lds(const uint4* kt, const uint4* vt, in
 #define AT_KEYS 64
 #define AT_CUS 256                   // compute units of the GPU
 #define AT_NT 1                      // column tiles per wave; 8 / AT_NT waves in a work-group
-// LDS row of key k of a tile (see am_block_lds), and the key of an LDS row
-__device__ __forceinline__ int at_lds_row(int k) {
-    return (k & 32) + ((k & 4) << 2) + ((k & 24) >> 1) + (k & 3);
-}
+// The key of a tile that LDS row `row` holds (see am_block_lds); key k lies in row
+// (k & 32) + ((k & 4) << 2) + ((k & 24) >> 1) + (k & 3).
 __device__ __forceinline__ int at_lds_key(int row) {
     return (row & 35) + ((row & 16) >> 2) + ((row & 12) << 1);
 }

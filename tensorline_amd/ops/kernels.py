@@ -580,6 +580,10 @@ def _key_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> tuple[int
     """(keys per split, number of splits) for ``num_seqs`` one-token sequences; (0, 1): no split."""
     base = (1 << max(num_seqs - 1, 0).bit_length()) * num_kv_heads
     split_len = 64 if base <= 8 else 128 if base <= 32 else 256 if base <= 128 else 512 if base <= 512 else 0
+    return _fit_key_splits(split_len, max_context)
+
+
+def _fit_key_splits(split_len: int, max_context: int) -> tuple[int, int]:
     if not split_len:
         return 0, 1
     while -(-max_context // split_len) > MAX_KEY_SPLITS:    # very long contexts: longer splits
@@ -662,18 +666,13 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         # together whatever the context length or the launch shape.  Pure decode steps split by the
         # batch size rounded up to a power of two (what a graph bucket pads to); steps with prompt
         # portions have enough columns and do not split.
-        split_len = 0
+        split_len, nsplit = 0, 1
         if split_keys is not None:
-            split_len = int(split_keys)
+            _check(int(split_keys) % 32 == 0, "paged_attention: a split is a multiple of 32 keys")
+            split_len, nsplit = _fit_key_splits(int(split_keys), plan.max_context)
         elif plan.decode_only:
-            split_len, _ = _key_splits(S, num_kv_heads, plan.max_context)
-        nsplit, split_blocks = 1, 1
-        if split_len:
-            _check(split_len % 32 == 0, "paged_attention: a split is a multiple of 32 keys")
-            while -(-plan.max_context // split_len) > MAX_KEY_SPLITS:    # very long contexts: longer splits
-                split_len *= 2
-            split_blocks = split_len // 32
-            nsplit = max(1, -(-plan.max_context // split_len))
+            split_len, nsplit = _key_splits(S, num_kv_heads, plan.max_context)
+        split_blocks = max(split_len // 32, 1)
         ws_o = ws_ml = None
         if nsplit > 1:
             ws = torch.empty(T * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
