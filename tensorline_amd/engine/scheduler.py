@@ -14,8 +14,13 @@ The decisions are those of the reference's ``BatchEngine._schedule`` (tensorline
    allow; a prompt longer than the budget is admitted in portions.  A request that does not fit
    even when nothing else runs fails with an error instead of waiting forever.
 
-Beyond the reference: a request whose prompt can never be held by the pool (even alone) is
-refused when it is added, so it cannot be admitted, preempt itself and be admitted again forever.
+Beyond the reference: a request that the pool can never hold, even alone, ends with
+:class:`RequestError` instead of being admitted, preempting itself and being admitted again
+forever (the reference only catches a first portion that does not fit, batch_engine.py:343-346).
+It is refused when added if its prompt is too long already; it fails at (re)admission if its
+prompt and generated tokens are; and it fails where it preempts itself while nothing else runs,
+which is how a request that outgrows the pool in the middle of a later portion or while decoding
+shows, whatever ``max_batched_tokens`` is.
 """
 from __future__ import annotations
 
@@ -112,6 +117,14 @@ class Scheduler:
         self.waiting.appendleft(req)
         self.preemptions += 1
 
+    def _fail_unholdable(self, req: Request) -> None:
+        """End a request (already out of both queues, its pages given back) that the pool cannot hold."""
+        req.done = True
+        req.error = RequestError(
+            f"request does not fit in the KV cache: its {len(req.tokens)} tokens and the next one need "
+            f"{self.cache.pages_for(len(req.tokens) + 1)} pages, the pool has {self.cache.num_blocks}")
+        self.failed.append(req)
+
     # ---- the plan ----------------------------------------------------------------------------
     def schedule(self) -> list[tuple[Request, int]]:
         budget = self.max_batched_tokens
@@ -132,12 +145,17 @@ class Scheduler:
                 plan = [(r, k) for r, k in plan if r is not victim]
                 if victim is req:
                     fits = False
+                    if not self.running:                     # it was alone and the whole pool is too small
+                        self._fail_unholdable(self.waiting.popleft())
                     break
             if fits:
                 plan.append((req, n))
                 budget -= n
         while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs:
             req = self.waiting[0]
+            if not self.cache.can_ever_hold(len(req.tokens) + 1, self.max_batched_tokens):
+                self._fail_unholdable(self.waiting.popleft())    # grew past the pool before it was preempted
+                continue
             if self.cache.add_request(req.rid) is None:
                 break                                        # no state slot free
             req.num_computed = self.cache.match_prefix(req.rid, req.tokens)
@@ -146,10 +164,7 @@ class Scheduler:
                 self._release(req)                           # drop prefix references while it waits
                 req.num_computed = 0
                 if not self.running:                         # can never fit, even alone
-                    self.waiting.popleft()
-                    req.done = True
-                    req.error = RequestError("request does not fit in the KV cache")
-                    self.failed.append(req)
+                    self._fail_unholdable(self.waiting.popleft())
                     continue
                 break                                        # wait for pages to come back
             self.waiting.popleft()

@@ -93,6 +93,27 @@ def test_oversized_request_errors_not_hangs(tiny, cpu_kernels):
         make_engine(d, max_model_len=8).add_request(list(range(8)))
 
 
+@pytest.mark.parametrize("budget, prompt_len, max_tokens", [(48, 60, 128), (16, 40, 100), (7, 62, 9)])
+def test_request_that_outgrows_the_pool_with_a_small_budget_errors(tiny, cpu_kernels, budget, prompt_len, max_tokens):
+    """The prompt fits, prompt plus generated tokens do not, and the token budget is smaller than
+    either: the first portion of a re-admission always fits, so only the request's whole length
+    tells that it can never run.  It must end with an error after a bounded number of steps."""
+    d, prompts, _ = tiny
+    eng = make_engine(d, num_blocks=8, block_size=8, max_batched_tokens=budget)
+    bystander = eng.add_request([1, 2, 3], SamplingParams(4, stop_token_ids=NO_STOP))
+    r = eng.add_request([t % 512 for t in range(prompt_len)], SamplingParams(max_tokens, stop_token_ids=NO_STOP))
+    steps = 0
+    while eng.has_work():
+        eng.step()
+        eng.cache.check()
+        steps += 1
+        assert steps <= prompt_len + 64 + 10, "the request is admitted and preempted again and again"
+    assert r.done and isinstance(r.error, RequestError) and "does not fit" in str(r.error)
+    assert len(r.tokens) <= 64 + 1                                # it got as far as the pool allows: 64 cached, one sampled
+    assert bystander.stats.finish_reason == "length" and bystander.error is None
+    assert eng.cache.all_free() and eng.counters()["requests_finished"].get("error") == 1
+
+
 def test_abort_frees_pages(tiny, cpu_kernels):
     d, prompts, _ = tiny
     eng = make_engine(d, block_size=4)
