@@ -10,6 +10,9 @@
 // [0, 1) given by the caller: the token is the first in index order whose running kept mass
 // exceeds u * kept_mass.
 #include "common.h"
+#include "argmax_static.h"
+
+#include <mutex>
 
 #define SM_THREADS 1024
 
@@ -101,6 +104,7 @@ __global__ void argmax_final_kernel(const float* __restrict__ pval, const int32_
 }
 
 #define AM_CHUNKS 64
+static_assert(AM_CHUNKS == TL_ARGMAX_STATIC_CHUNKS, "the static buffer is sized for the chunking of tl_argmax");
 // scratch: room for R * 64 floats and R * 64 int32 when V > 8192 (may be null otherwise)
 extern "C" int tl_argmax(const float* logits, int ld, int R, int V, int32_t* out, float* scratch_val,
                          int32_t* scratch_idx, hipStream_t stream) {
@@ -118,6 +122,52 @@ extern "C" int tl_argmax(const float* logits, int ld, int R, int V, int32_t* out
     hipLaunchKernelGGL(argmax_final_kernel, dim3(R), dim3(TL_WAVE), 0, stream, scratch_val, scratch_idx, nch, out);
     TL_CHECK_LAUNCH("tl_argmax");
     return 0;
+}
+
+// ---- arg-max without an allocation ------------------------------------------------------------
+// The partial results of wide rows live in this array: TL_ARGMAX_STATIC_MAX_ROWS * 64 floats (the
+// chunks' best values), then as many int32 (their indices).  In host code the array's name is a
+// stand-in, not a device address: hipGetSymbolAddress gives the address, once per GPU, because
+// every GPU holds a copy of its own.  Kernels get that address as an argument.
+static __device__ __align__(256) unsigned char scratch[TL_ARGMAX_STATIC_BYTES];
+
+#define TL_MAX_DEVICES 64
+static void* g_scratch_ptr[TL_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int argmax_static_ptr(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return tl_fail("tl_argmax_static: hipGetDevice failed: %s", hipGetErrorString(e));
+    TL_CHECK_ARG(dev >= 0 && dev < TL_MAX_DEVICES, "tl_argmax_static: device %d is outside [0, %d)", dev, TL_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return tl_fail("tl_argmax_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" int tl_argmax_static_setup(void) {
+    void* p = nullptr;
+    return argmax_static_ptr(&p);
+}
+
+extern "C" int tl_argmax_static(const float* logits, int ld, int R, int V, int32_t* out, hipStream_t stream) {
+    TL_CHECK_ARG(R >= 0 && V > 0 && ld >= V, "tl_argmax_static: bad sizes R=%d V=%d ld=%d", R, V, ld);
+    TL_CHECK_ARG(R <= TL_ARGMAX_STATIC_MAX_ROWS, "tl_argmax_static: %d rows exceed the %d the static buffer holds", R,
+                 TL_ARGMAX_STATIC_MAX_ROWS);
+    TL_CHECK_ARG(logits && out, "tl_argmax_static: null logits or output");
+    if (R == 0) return 0;
+    void* base = nullptr;
+    if (int rc = argmax_static_ptr(&base)) return rc;
+    float* pval = (float*)base;
+    int32_t* pidx = (int32_t*)((unsigned char*)base + (size_t)TL_ARGMAX_STATIC_MAX_ROWS * TL_ARGMAX_STATIC_CHUNKS * 4);
+    return tl_argmax(logits, ld, R, V, out, pval, pidx, stream);
 }
 
 // ---- temperature / top-p sampling ---------------------------------------------------------------
