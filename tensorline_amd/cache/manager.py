@@ -26,7 +26,7 @@ from typing import Sequence
 import numpy as np
 import torch
 
-from tensorline_amd.cache.allocator import BlockAllocator, block_hash
+from tensorline_amd.cache.allocator import PagePool, page_key
 from tensorline_amd.parts.spec import CacheNeed, ScheduleEntry, StateNeed
 
 _TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
@@ -36,7 +36,7 @@ _TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": 
 class CacheGroup:
     need: CacheNeed
     entries: list[int]                       # schedule entries with storage in this group
-    allocator: BlockAllocator
+    allocator: PagePool
     k: dict[int, torch.Tensor] = field(default_factory=dict)
     v: dict[int, torch.Tensor] = field(default_factory=dict)
 
@@ -86,7 +86,7 @@ class CacheManager:
             if g is None:
                 g = len(self.groups)
                 by_need[need] = g
-                self.groups.append(CacheGroup(need, [], BlockAllocator(num_blocks, prefix_caching=False)))
+                self.groups.append(CacheGroup(need, [], PagePool(num_blocks, share_prefixes=False)))
             self.groups[g].entries.append(i)
             self.group_of_entry[i] = g
             self.storage_entry[i] = i
@@ -110,7 +110,7 @@ class CacheManager:
         self.prefix_caching = bool(prefix_caching) and len(self.groups) == 1 and self.groups[0].window == 0 \
             and not self.has_state
         if self.prefix_caching:
-            self.groups[0].allocator.prefix_caching = True
+            self.groups[0].allocator.share_prefixes = True
 
         if allocate_storage:
             for g in self.groups:
@@ -149,7 +149,7 @@ class CacheManager:
 
     def all_free(self) -> bool:
         """No page and no slot is held (reference invariant: tests/test_batching.py:80)."""
-        return all(g.allocator.num_free == g.allocator.num_blocks for g in self.groups) \
+        return all(g.allocator.num_free == g.allocator.num_pages for g in self.groups) \
             and len(self._free_slots) == self.max_requests and not self._requests
 
     def can_ever_hold(self, tokens: int, step_tokens: int) -> bool:
@@ -222,7 +222,7 @@ class CacheManager:
             return False
         for gi, (n, g, t) in enumerate(zip(needs, self.groups, req.tables)):
             if n:
-                got = g.allocator.allocate(n)
+                got = g.allocator.take(n)
                 assert got is not None
                 t.extend(got)
                 req.arrays[gi] = None
@@ -249,7 +249,7 @@ class CacheManager:
                     back.append(req.tables[gi][lp])
                     req.tables[gi][lp] = -1
             if back:
-                g.allocator.free(back)
+                g.allocator.give_back(back)
                 given += len(back)
                 req.arrays[gi] = None
             req.trimmed[gi] = max(req.trimmed[gi], upto_page)
@@ -259,7 +259,7 @@ class CacheManager:
         """Give back every page and the state slot of a request."""
         req = self._requests.pop(rid)
         for g, t in zip(self.groups, req.tables):
-            g.allocator.free([b for b in t if b >= 0])
+            g.allocator.give_back([b for b in t if b >= 0])
         self._free_slots.append(req.state_slot)
 
     def live_requests(self) -> list:
@@ -279,15 +279,15 @@ class CacheManager:
         alloc, bs, parent = self.groups[0].allocator, self.page_size, None
         for i in range(len(tokens) // bs):
             content = (parent, tuple(tokens[i * bs:(i + 1) * bs]))
-            h = hash(content)
-            blk = alloc.lookup(h, content)
+            h = page_key(*content)
+            blk = alloc.revive(h, content)
             if blk is None:
                 break
             table.append(blk)
             req.hashes.append(h)
             parent = h
         if table and len(table) * bs == len(tokens):
-            alloc.free([table.pop()])
+            alloc.give_back([table.pop()])
             req.hashes.pop()
         req.arrays[0] = None
         return len(table) * bs
@@ -302,10 +302,9 @@ class CacheManager:
         while len(req.hashes) < min(computed, len(tokens)) // bs:
             i = len(req.hashes)
             content = (req.hashes[-1] if i else None, tuple(tokens[i * bs:(i + 1) * bs]))
-            h = hash(content)
-            assert h == block_hash(content[0], content[1])
+            h = page_key(*content)
             req.hashes.append(h)
-            alloc.register(table[i], h, content)
+            alloc.publish(table[i], h, content)
 
     # ---- views for the step function -------------------------------------------------------
     def storage(self, entry: int) -> tuple[torch.Tensor | None, torch.Tensor | None]:

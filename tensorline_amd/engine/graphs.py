@@ -28,14 +28,6 @@ from tensorline_amd.engine.batch import StepEntry
 from tensorline_amd.engine.runner import ModelRunner
 
 
-def _pow2_upto(limit: int) -> list[int]:
-    out, b = [], 1
-    while b < limit:
-        out.append(b)
-        b *= 2
-    return out + [limit]
-
-
 class _Captured:
     def __init__(self, graph, dev, host, logits, packed):
         self.graph, self.dev, self.host, self.logits, self.packed = graph, dev, host, logits, packed
@@ -49,7 +41,8 @@ class _Captured:
 class GraphRunner(ModelRunner):
     def __init__(self, model, cache: CacheManager, max_batch: int, max_blocks_per_seq: int):
         super().__init__(model, cache)
-        self.batch_buckets = _pow2_upto(max_batch)
+        # batch sizes a graph exists for: the powers of two below max_batch, and max_batch itself
+        self.batch_buckets = sorted({1 << k for k in range(max(max_batch - 1, 0).bit_length())} | {max_batch})
         self.max_blocks = max_blocks_per_seq
         self.graphs: dict[int, _Captured] = {}
         self.graph_replays = 0

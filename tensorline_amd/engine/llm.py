@@ -133,6 +133,9 @@ class LLM:
                             yield delta
             if req.error is not None:
                 raise req.error
+            tail = detok.flush() if detok is not None else ""
+            if tail:                                         # the output ended inside a character
+                yield tail
         finally:
             self.engine.abort(req)
 

@@ -6,45 +6,89 @@ import pytest
 import torch
 from hypothesis import given, settings, strategies as st
 
-from tensorline_amd.cache.allocator import BlockAllocator, block_hash
+from tensorline_amd.cache.allocator import PagePool, page_key
 from tensorline_amd.cache.manager import CacheManager
 from tensorline_amd.parts.spec import CacheNeed, ScheduleEntry, StateNeed
 
 
 def test_allocator_refcount_lru_and_eviction():
     # the sequence of the reference's own test (tests/test_prefix_cache.py:8-22)
-    a = BlockAllocator(4)
-    x = a.allocate(2)
-    h0 = block_hash(None, [1, 2])
-    a.register(x[0], h0)
-    a.free(x)
+    a = PagePool(4)
+    x = a.take(2)
+    h0 = page_key(None, [1, 2])
+    a.publish(x[0], h0)
+    a.give_back(x)
     assert a.num_free == 4 and a.num_cached == 1          # freed but still cached
-    assert a.lookup(h0) == x[0] and a.num_free == 3       # revived from the free list
-    assert a.lookup(h0) == x[0]                           # shared: two references
-    a.free([x[0]])
+    assert a.revive(h0) == x[0] and a.num_free == 3       # revived from the free list
+    assert a.revive(h0) == x[0]                           # shared: two references
+    a.give_back([x[0]])
     assert a.num_free == 3                                # still referenced once
-    a.free([x[0]])
+    a.give_back([x[0]])
     assert a.num_free == 4
-    a.allocate(4)                                         # memory pressure evicts it
-    assert a.num_cached == 0 and a.lookup(h0) is None
+    a.take(4)                                         # memory pressure evicts it
+    assert a.num_cached == 0 and a.revive(h0) is None
 
 
 def test_allocator_details():
-    assert block_hash(block_hash(None, [1]), [2]) != block_hash(block_hash(None, [9]), [2])   # chained over the prefix
-    a = BlockAllocator(3)
-    assert a.allocate(4) is None and a.num_free == 3      # all or nothing
-    x = a.allocate(3)
-    a.free([x[1]])
+    assert page_key(page_key(None, [1]), [2]) != page_key(page_key(None, [9]), [2])   # chained over the prefix
+    a = PagePool(3)
+    assert a.take(4) is None and a.num_free == 3      # all or nothing
+    x = a.take(3)
+    a.give_back([x[1]])
     with pytest.raises(AssertionError, match="double free"):
-        a.free([x[1]])
-    a.free([x[0], x[2]])                                  # reversed: the tail page is handed out first
-    assert a.allocate(1) == [x[1]] and a.allocate(1) == [x[2]]
-    b = BlockAllocator(2)
-    y = b.allocate(1)
-    b.register(y[0], 5, content=(None, (1, 2)))
-    assert b.lookup(5, content=(None, (9, 9))) is None    # same hash, other tokens: no hit
-    assert b.lookup(5, content=(None, (1, 2))) == y[0]
+        a.give_back([x[1]])
+    a.give_back([x[0], x[2]])                                  # reversed: the tail page is handed out first
+    assert a.take(1) == [x[1]] and a.take(1) == [x[2]]
+    b = PagePool(2)
+    y = b.take(1)
+    b.publish(y[0], 5, contents=(None, (1, 2)))
+    assert b.revive(5, contents=(None, (9, 9))) is None    # same hash, other tokens: no hit
+    assert b.revive(5, contents=(None, (1, 2))) == y[0]
     b.check({y[0]: 2})
+
+
+@settings(max_examples=60, deadline=None)
+@given(st.lists(st.tuples(st.sampled_from(["take", "give", "publish", "revive"]), st.integers(0, 7)), max_size=80))
+def test_pool_hands_out_in_the_order_of_return_whatever_leaves_the_middle_of_the_queue(ops):
+    """The pool against a plain list as the queue: same pages in the same order, a published page
+    found while it waits and gone once it is handed out for something else."""
+    n = 6
+    pool, queue, holders, key_of = PagePool(n), list(range(n)), [0] * n, {}
+    held: list[int] = []
+    for op, x in ops:
+        if op == "take":
+            k = x % 4
+            got = pool.take(k)
+            if k > len(queue):
+                assert got is None
+            else:
+                want, queue = queue[:k], queue[k:]
+                assert got == want
+                for p in want:
+                    holders[p] = 1
+                    key_of = {key: q for key, q in key_of.items() if q != p}
+                held += want
+        elif op == "give" and held:
+            p = held.pop(x % len(held))
+            pool.give_back([p])
+            holders[p] -= 1
+            if holders[p] == 0:
+                queue.append(p)
+        elif op == "publish" and held:
+            p = held[x % len(held)]
+            if x not in key_of and p not in key_of.values():
+                key_of[x] = p
+            pool.publish(p, x)
+        elif op == "revive":
+            got = pool.revive(x)
+            assert got == key_of.get(x)
+            if got is not None:
+                if holders[got] == 0:
+                    queue.remove(got)
+                holders[got] += 1
+                held.append(got)
+        pool.check({p: c for p, c in enumerate(holders) if c})
+        assert pool.num_free == len(queue) and pool.num_cached == len(key_of)
 
 
 def manager(needs, schedule=None, states=None, **kw):

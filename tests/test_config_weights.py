@@ -131,6 +131,36 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(folder):
     assert "missing tensors (2)" in msg and "unexpected tensors (1)" in msg and "wrong shapes (1)" in msg
 
 
+def test_wrong_dtypes_are_an_error_and_extra_tensors_alone_a_warning(folder):
+    d, _ = folder
+    path = os.path.join(d, "model.safetensors")
+    good = load_file(path)
+    raw = dict(good)
+    raw["rotary.inv_freq"] = torch.zeros(4)                                  # something the model does not know
+    save_file(raw, path)
+    with pytest.warns(UserWarning, match="rotary.inv_freq"):
+        model, _ = load_model(d, "float32", "cpu")
+    assert torch.equal(model.embed_table, good["model.embed_tokens.weight"].float())
+    # integer and 64-bit tensors under the names of float weights: one error names each, and the extra tensor too
+    raw["model.layers.1.mlp.down_proj.weight"] = torch.zeros_like(good["model.layers.1.mlp.down_proj.weight"], dtype=torch.int64)
+    raw["model.norm.weight"] = good["model.norm.weight"].double()
+    raw["model.layers.0.self_attn.v_proj.bias"] = good["model.layers.0.self_attn.v_proj.bias"].to(torch.int8)
+    save_file(raw, path)
+    with pytest.raises(WeightError) as e:
+        load_model(d, "bfloat16", "cpu")
+    err = e.value
+    assert sorted(w.split(":")[0] for w in err.wrong_dtype) == [
+        "model.layers.0.self_attn.v_proj.bias", "model.layers.1.mlp.down_proj.weight", "model.norm.weight"]
+    assert "I64" in str(err) and "F64" in str(err) and "I8" in str(err) and "wrong dtypes (3)" in str(err)
+    assert err.unexpected == ["rotary.inv_freq"] and not err.missing and not err.wrong_shape
+    # half precision is a float dtype: accepted
+    raw = dict(good)
+    raw["model.norm.weight"] = good["model.norm.weight"].half()
+    save_file(raw, path)
+    load_model(d, "float32", "cpu")
+    save_file(good, path)
+
+
 def test_tied_head(tmp_path):
     cfg = Qwen2Config.from_dict(helpers.TINY_A)
     d = write_random_model(cfg, str(tmp_path / "tied"), seed=1)

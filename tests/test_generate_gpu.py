@@ -127,7 +127,7 @@ def test_graph_decode_matches_eager_and_isolates_padding(folder_b):
     for c in (ce, cg):
         for i, s in enumerate(seqs):
             c.add_request(i)
-        c.groups[0].allocator.allocate(5)             # shift the ids so tables are not 0, 1, 2, ...
+        c.groups[0].allocator.take(5)             # shift the ids so tables are not 0, 1, 2, ...
         for i, s in enumerate(seqs):
             assert c.grow(i, len(s) + 21)
         assert all(bystander not in c.table(i) for i in range(3))
