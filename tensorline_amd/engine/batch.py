@@ -37,6 +37,9 @@ class AttentionPlan:
     # In a step that mixes prompt portions with one-token sequences: the indices of the latter
     # (also on the device, ``StepContext.single_seqs``), so that they can be given to a kernel of their own.
     singles: list[int] = field(default_factory=list)
+    # The longest context the engine will ever run, if the caller knows it (0: unknown).  Choices
+    # that must be the same in every step of an engine (the length of a key split) are made for it.
+    fit_context: int = 0
 
 
 @dataclass

@@ -13,6 +13,7 @@ import time
 
 from tensorline_amd.cache.manager import CacheManager
 from tensorline_amd.engine.batch import StepEntry
+from tensorline_amd.engine.metrics import EngineMetrics
 from tensorline_amd.engine.runner import ModelRunner
 from tensorline_amd.engine.scheduler import Request, Scheduler
 from tensorline_amd.sampling.params import GenStats, SamplingParams
@@ -29,10 +30,9 @@ class InferenceEngine:
         self.default_stops = set(default_stops or ())
         self._ids = itertools.count()
         self._seed_source = random.Random(0)
-        # counters (reference: batch_engine.py:119-125, metrics.py:37-43)
+        # counters and distributions (reference: batch_engine.py:119-125, metrics.py:37-43)
         self.steps = 0
-        self.tokens_generated = 0
-        self.requests_finished: dict[str, int] = {}
+        self.metrics = EngineMetrics()
 
     # ---- requests ------------------------------------------------------------------------------
     def add_request(self, prompt_tokens: list[int], params: SamplingParams | None = None,
@@ -55,9 +55,18 @@ class InferenceEngine:
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 
+    @property
+    def tokens_generated(self) -> int:
+        return self.metrics.tokens_generated
+
+    @property
+    def requests_finished(self) -> dict:
+        return self.metrics.requests_finished
+
     def _count(self, req: Request) -> None:
+        """A request ended: by its reason, and its whole time if it ran to a stop or its length."""
         reason = "error" if req.error is not None else req.stats.finish_reason
-        self.requests_finished[reason] = self.requests_finished.get(reason, 0) + 1
+        self.metrics.finished(reason, req.stats.total_s if reason in ("stop", "length") else None)
 
     # ---- one iteration -------------------------------------------------------------------------
     def step(self) -> list[tuple[Request, int | None]]:
@@ -90,12 +99,16 @@ class InferenceEngine:
                 events.append((req, None))
             raise
         self.steps += 1
+        self.metrics.batch_size.observe(len(plan))
         sched.computed(plan)
         now = time.perf_counter()
         for req, tok in zip(sampled, toks):
+            first = req.num_generated == 0 and req.stats.ttft_s == 0.0
             if sched.accept(req, int(tok), now):
-                self.tokens_generated += 1
+                self.metrics.tokens_generated += 1
                 events.append((req, int(tok)))
+            if first:
+                self.metrics.ttft_s.observe(req.stats.ttft_s)
             if req.done:
                 self._count(req)
                 events.append((req, None))
@@ -106,8 +119,9 @@ class InferenceEngine:
             self.step()
 
     def counters(self) -> dict:
-        s = self.scheduler
+        """Totals since the engine started, and the distributions of time to first token, whole
+        request time (seconds) and sequences per step."""
+        s, m = self.scheduler, self.metrics.as_dict()
         return {"steps": self.steps, "preemptions": s.preemptions, "max_running_seen": s.max_running_seen,
                 "prompt_tokens_total": s.prompt_tokens_total, "prefix_hit_tokens": s.prefix_hit_tokens,
-                "tokens_generated": self.tokens_generated, "requests_finished": dict(self.requests_finished),
-                "graph_replays": getattr(self.runner, "graph_replays", 0)}
+                "graph_replays": getattr(self.runner, "graph_replays", 0), **m}

@@ -44,6 +44,7 @@ class GraphRunner(ModelRunner):
         # batch sizes a graph exists for: the powers of two below max_batch, and max_batch itself
         self.batch_buckets = sorted({1 << k for k in range(max(max_batch - 1, 0).bit_length())} | {max_batch})
         self.max_blocks = max_blocks_per_seq
+        self.fit_context = max_blocks_per_seq * cache.page_size   # eager steps split keys as the graphs do
         self.graphs: dict[int, _Captured] = {}
         self.graph_replays = 0
         self.pool = None
@@ -84,7 +85,7 @@ class GraphRunner(ModelRunner):
     @torch.inference_mode()
     def _capture(self, B: int) -> _Captured:
         packed = self._padding_batch(B)
-        packed.plan.max_context = self.max_blocks * self.cache.page_size
+        packed.plan.max_context = packed.plan.fit_context = self.fit_context
         packed.plan.decode_only = True
         n = packed.data.size
         dev = torch.empty(n, dtype=torch.int32, device=self.device)

@@ -72,6 +72,8 @@ class LLM:
         self.engine = InferenceEngine(self.model, self.cache, max_num_seqs=ec.max_num_seqs,
                                       max_batched_tokens=ec.max_batched_tokens, max_model_len=ec.max_model_len,
                                       default_stops=set(self.model.spec.eos_token_ids), runner=runner)
+        # with or without graphs, every step makes the choices that depend on the longest context alike
+        self.engine.runner.fit_context = -(-ec.max_model_len // ec.block_size) * ec.block_size
 
     def _size_cache(self) -> int:
         """Pages from ``kv_cache_gb`` or from a share of free memory (batch_engine.py:89-97)."""

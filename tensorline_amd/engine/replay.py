@@ -37,15 +37,25 @@ class TraceError(RuntimeError):
 class TraceSession:
     """Live requests of a trace and the cache they share."""
 
-    def __init__(self, model, max_tokens: int, page_size: int = 16, max_requests: int = 8):
+    def __init__(self, model, max_tokens: int, page_size: int = 16, max_requests: int = 8, graphs: bool = False):
+        """``max_tokens``: the most tokens live requests hold at any time (each request's count
+        rounded up to 64); ``max_requests``: the most requests live at a time.  ``graphs``: steps
+        that are pure decoding replay a HIP graph, as the engine's do, instead of running eagerly."""
         if ROUND_TOKENS % page_size:
             raise ValueError(f"page size {page_size} must divide {ROUND_TOKENS}")
+        if max_requests <= 0:
+            raise ValueError("max_requests must be positive")
         num_blocks = max(1, -(-int(max_tokens) // page_size))
         self.model = model
         self.cache = CacheManager(model.cache_needs(), model.schedule, model.state_needs(), page_size=page_size,
                                   num_blocks=num_blocks, max_requests=max_requests, dtype=model.dtype,
                                   device=model.device, prefix_caching=False)
-        self.runner = ModelRunner(model, self.cache)
+        if graphs:
+            from tensorline_amd.engine.graphs import GraphRunner
+            # one request can hold the whole pool at most: that bounds every page table
+            self.runner = GraphRunner(model, self.cache, max_batch=max_requests, max_blocks_per_seq=num_blocks)
+        else:
+            self.runner = ModelRunner(model, self.cache)
         self.computed: dict[str, int] = {}
 
     def step(self, entries: list[dict], end: list[str] | tuple = ()) -> np.ndarray | None:
@@ -62,7 +72,7 @@ class TraceSession:
                 raise TraceError(f"request {rid!r} brings no tokens")
             if rid not in self.computed:
                 if self.cache.add_request(rid) is None:
-                    raise TraceError(f"more than {self.cache.max_requests} requests are live at once")
+                    raise TraceError(f"more than {self.cache.max_requests} requests are live at once (--max-requests)")
                 self.computed[rid] = 0
             start = self.computed[rid]
             if not self.cache.grow(rid, start + len(tokens)):
@@ -77,7 +87,7 @@ class TraceSession:
                 self.computed[b.rid] += len(b.tokens)
                 self.cache.trim(b.rid, self.computed[b.rid])
             if out.shape[0]:
-                logits = out.to(torch.float32).cpu().numpy()
+                logits = out.to(torch.float32).cpu().numpy()     # a copy: a replayed graph writes its logits in place
         for rid in end:
             rid = str(rid)
             if rid in self.computed:
@@ -94,6 +104,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64); sizes the cache")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
+    ap.add_argument("--max-requests", type=int, default=8, help="most requests live at any time")
+    ap.add_argument("--graphs", action="store_true", help="replay HIP graphs for steps that only decode, as serving does")
     ap.add_argument("--device", default="cuda:0")
     return ap
 
@@ -108,7 +120,8 @@ def main(argv=None, stdin=None, stdout=None) -> int:
     kernels.require_gpu(args.device)
     os.makedirs(args.out, exist_ok=True)
     model, _ = load_model(args.model, args.dtype, args.device)
-    session = TraceSession(model, args.max_tokens, page_size=args.block_size)
+    session = TraceSession(model, args.max_tokens, page_size=args.block_size, max_requests=args.max_requests,
+                           graphs=args.graphs)
     for line in stdin:
         line = line.strip()
         if not line:

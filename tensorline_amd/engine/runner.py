@@ -27,6 +27,7 @@ class ModelRunner:
         self._host: torch.Tensor | None = None       # pinned staging for the step's metadata
         self._dev: torch.Tensor | None = None
         self.steps = 0
+        self.fit_context = 0          # the longest context this runner's engine allows, if it says so
 
     # ---- metadata ------------------------------------------------------------------------
     def _upload(self, data: np.ndarray) -> torch.Tensor:
@@ -46,9 +47,11 @@ class ModelRunner:
         ngroups = len(cache.groups)
         tables = [[cache.table_array(e.rid, g) for g in range(ngroups)] for e in entries]
         slots = [cache.state_slot(e.rid) for e in entries]
-        return pack_batch(entries, tables, slots, cache.page_size, ngroups, cache.scratch_page,
-                          self.model.vocab_size, pad_seqs=pad_seqs, pad_nb=pad_nb, scratch_slot=cache.scratch_slot,
-                          windowed=[g.window > 0 for g in cache.groups])
+        packed = pack_batch(entries, tables, slots, cache.page_size, ngroups, cache.scratch_page,
+                            self.model.vocab_size, pad_seqs=pad_seqs, pad_nb=pad_nb, scratch_slot=cache.scratch_slot,
+                            windowed=[g.window > 0 for g in cache.groups])
+        packed.plan.fit_context = self.fit_context
+        return packed
 
     def context(self, packed: PackedBatch, dev: torch.Tensor) -> tuple[StepContext, list[LayerCache]]:
         def view(name: str) -> torch.Tensor:

@@ -576,17 +576,21 @@ def _singles_get_own_launch(plan, singles: list[int], num_heads: int, num_kv_hea
     return walk_us > portions_us + 9 + stream_us + 5
 
 
-def _key_splits(num_seqs: int, num_kv_heads: int, max_context: int) -> tuple[int, int]:
+def _key_splits(num_seqs: int, num_kv_heads: int, max_context: int, fit_context: int = 0) -> tuple[int, int]:
     """(keys per split, number of splits) for ``num_seqs`` one-token sequences; (0, 1): no split."""
     base = (1 << max(num_seqs - 1, 0).bit_length()) * num_kv_heads
     split_len = 64 if base <= 8 else 128 if base <= 32 else 256 if base <= 128 else 512 if base <= 512 else 0
-    return _fit_key_splits(split_len, max_context)
+    return _fit_key_splits(split_len, max_context, fit_context)
 
 
-def _fit_key_splits(split_len: int, max_context: int) -> tuple[int, int]:
+def _fit_key_splits(split_len: int, max_context: int, fit_context: int = 0) -> tuple[int, int]:
+    """Splits get longer where there would be more than the merge kernel takes.  Their length is
+    fitted to ``fit_context``, the longest context the engine ever runs, where the caller knows it
+    (else to this step's longest): then every step of an engine, eager or replayed from a graph
+    captured for the longest context, sums the same runs of keys together."""
     if not split_len:
         return 0, 1
-    while -(-max_context // split_len) > MAX_KEY_SPLITS:    # very long contexts: longer splits
+    while -(-max(max_context, fit_context) // split_len) > MAX_KEY_SPLITS:
         split_len *= 2
     return split_len, max(1, -(-max_context // split_len))
 
@@ -644,7 +648,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if singles and route_singles is not False:
             _i32(single_seqs, "single_seqs", len(singles))
             ctx1 = max([plan.starts[s] + 1 for s in singles if s < len(plan.starts)] + [1])
-            split_len, nsplit = _key_splits(len(singles), num_kv_heads, ctx1)
+            split_len, nsplit = _key_splits(len(singles), num_kv_heads, ctx1, plan.fit_context)
             if route_singles or (route_singles is None and nsplit > 1 and _singles_get_own_launch(
                     plan, singles, num_heads, num_kv_heads, head_dim, int(window))):
                 nt1 = 1 if G <= 16 else 2
@@ -669,9 +673,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         split_len, nsplit = 0, 1
         if split_keys is not None:
             _check(int(split_keys) % 32 == 0, "paged_attention: a split is a multiple of 32 keys")
-            split_len, nsplit = _fit_key_splits(int(split_keys), plan.max_context)
+            split_len, nsplit = _fit_key_splits(int(split_keys), plan.max_context, plan.fit_context)
         elif plan.decode_only:
-            split_len, nsplit = _key_splits(S, num_kv_heads, plan.max_context)
+            split_len, nsplit = _key_splits(S, num_kv_heads, plan.max_context, plan.fit_context)
         split_blocks = max(split_len // 32, 1)
         ws_o = ws_ml = None
         if nsplit > 1:

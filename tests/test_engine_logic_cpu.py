@@ -31,3 +31,23 @@ def test_cuttings_match_plain(setup, cut, cpu_kernels):
         np.testing.assert_allclose(got[key], want[key], atol=2e-5, rtol=1e-4, err_msg=str(key))
     assert session.cache.all_free()
     session.cache.check()
+
+
+def test_more_live_requests_than_the_default_when_asked_for(setup, cpu_kernels):
+    """The number of requests live at a time is the caller's to give: ten at once with room for
+    twelve, and a clear error where the room is too small."""
+    from tensorline_amd.engine.replay import TraceError
+    name, d, reqs, want = setup
+    if name != "A":
+        pytest.skip("one configuration is enough")
+    model, _ = load_model(d, "float32", "cpu")
+    toks = reqs["r1"]
+    ids = [f"x{i}" for i in range(10)]
+    session = TraceSession(model, 64 * len(ids), page_size=16, max_requests=12)
+    got = session.step([{"id": i, "tokens": toks, "want": [len(toks) - 1]} for i in ids], end=ids[:5])
+    for row in got:
+        np.testing.assert_allclose(row, want[("r1", len(toks) - 1)], atol=2e-5, rtol=1e-4)
+    assert len(session.cache.live_requests()) == 5
+    small = TraceSession(model, 64 * len(ids), page_size=16, max_requests=4)
+    with pytest.raises(TraceError, match="max-requests"):
+        small.step([{"id": i, "tokens": toks, "want": []} for i in ids])

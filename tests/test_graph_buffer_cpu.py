@@ -83,3 +83,18 @@ def test_in_place_update_is_off_for_windowed_caches():
     cap = _cap(runner, [StepEntry("a", [1], 5, [0])])
     cache.grow("a", 7)
     assert not runner._advance(cap, [StepEntry("a", [1], 6, [0])])
+
+
+def test_key_splits_are_fitted_to_the_longest_context_the_engine_runs():
+    """A graph is captured for the longest context, an eager step sees the real one: both must cut
+    the keys into the same runs, so the length of a split follows the engine's limit where it is
+    known and only the number of splits follows the step."""
+    from tensorline_amd.ops.kernels import MAX_KEY_SPLITS, _fit_key_splits, _key_splits
+    assert _key_splits(1, 4, 3000) == (64, 47)
+    assert _key_splits(1, 4, 3000, fit_context=4096) == (64, 47)
+    long = 64 * MAX_KEY_SPLITS * 2                        # twice what 1,024 splits of 64 keys cover
+    graph = _key_splits(1, 4, long, fit_context=long)
+    eager = _key_splits(1, 4, 3000, fit_context=long)
+    assert graph == (128, MAX_KEY_SPLITS) and eager == (128, 24)
+    assert _key_splits(1, 4, 3000) == (64, 47)            # without the hint only the step's own context counts
+    assert _fit_key_splits(0, 10 ** 6, 10 ** 7) == (0, 1)

@@ -201,3 +201,36 @@ def test_head_of_line_waits_and_is_admitted_later():
     assert a.done and s.cache.all_free()
     plan = s.schedule()
     assert [(r.rid, n) for r, n in plan] == [(1, 8)]
+
+
+def test_distribution_buckets_and_quantiles():
+    from tensorline_amd.engine.metrics import BATCH_BOUNDS, Distribution
+    d = Distribution(BATCH_BOUNDS)
+    assert d.as_dict()["count"] == 0 and d.quantile(0.5) == 0.0
+    for v in [1, 1, 2, 3, 4, 64, 65, 500]:
+        d.observe(v)
+    b = d.as_dict()["buckets"]
+    # a value on a bound belongs to the bucket that bound closes (the reference's bisect_left rule)
+    assert (b["le_1"], b["le_2"], b["le_4"], b["le_8"], b["le_64"], b["le_128"], b["above"]) == (2, 1, 2, 0, 1, 1, 1)
+    assert d.count == 8 and d.total == 640 and d.smallest == 1 and d.largest == 500
+    assert 2 <= d.quantile(0.5) <= 4 and d.quantile(1.0) == 500 and d.quantile(0.0) == 1
+    with pytest.raises(ValueError):
+        Distribution((2, 1))
+
+
+def test_engine_reports_distributions_of_latency_and_batch_size(tiny, cpu_kernels):
+    d, prompts, want = tiny
+    eng = make_engine(d, max_num_seqs=3)
+    reqs = [eng.add_request(p, SamplingParams(5, stop_token_ids=NO_STOP)) for p in prompts[:6]]
+    gone = eng.add_request(prompts[6], SamplingParams(50, stop_token_ids=NO_STOP))
+    eng.step()
+    eng.abort(gone)
+    eng.run_until_done()
+    c = eng.counters()
+    assert c["tokens_generated"] == 6 * 5 and c["requests_finished"] == {"length": 6, "abort": 1}
+    assert c["ttft_s"]["count"] == 6 and c["e2e_s"]["count"] == 6           # the aborted one gave no token
+    assert c["e2e_s"]["min"] >= c["ttft_s"]["min"] > 0
+    assert abs(c["e2e_s"]["sum"] - sum(r.stats.total_s for r in reqs)) < 1e-9
+    bs = c["batch_size"]
+    assert bs["count"] == c["steps"] and bs["max"] == 3 == c["max_running_seen"]
+    assert sum(bs["buckets"].values()) == bs["count"] and bs["buckets"]["le_4"] > 0
