@@ -1,0 +1,150 @@
+"""A model with the layer sizes of Qwen2.5-7B (hidden 3584, 28 query and 4 key/value heads of 128,
+feed-forward 18944, vocabulary 152064) and 2 of its 28 layers, against the plain implementation:
+the branches that only real sizes take (the wide head, products cut into shares of K, groups of
+seven query heads, hundreds of column groups in prompt attention, the 17-to-64-row kernels and
+graph buckets above 16 rows) as a whole model, in 32-bit and in bfloat16, in every way of cutting
+(analogue of the reference's tests/test_batching.py:48-64 at a size its own tests never reach)."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers, plain
+
+pytestmark = pytest.mark.gpu
+
+SHAPE_7B_2_LAYERS = dict(
+    architectures=["Qwen2ForCausalLM"], vocab_size=152064, hidden_size=3584, intermediate_size=18944,
+    num_hidden_layers=2, num_attention_heads=28, num_key_value_heads=4, head_dim=128, rope_theta=1000000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768)
+LENGTHS = {"tiny": 3, "short": 70, "mid": 200, "long": 2100}
+LIMIT = {"float32": 1e-5, "bfloat16": 2e-2}
+PAGE = 16
+
+
+def kept_positions(n: int) -> list[int]:
+    """Where logits are compared: the first tokens, both sides of page and tile edges, a sparse
+    sweep, and the last 40 (all of them for short requests)."""
+    if n <= 256:
+        return list(range(n))
+    keep = {0, 1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 1023, 1024, 2047, 2048}
+    keep |= set(range(0, n, 97)) | set(range(n - 40, n))
+    return sorted(p for p in keep if p < n)
+
+
+@pytest.fixture(scope="module")
+def oracle(tmp_path_factory):
+    from tensorline_amd.config import Qwen2Config
+    from tensorline_amd.weights import write_random_model
+    d = write_random_model(Qwen2Config.from_dict(SHAPE_7B_2_LAYERS), str(tmp_path_factory.mktemp("real_sizes")), seed=17)
+    w, cfg = plain.load_folder(d)
+    rng = random.Random(23)
+    reqs = {name: [rng.randrange(cfg["vocab_size"]) for _ in range(n)] for name, n in LENGTHS.items()}
+    want = {}
+    with torch.inference_mode():
+        for name, toks in reqs.items():
+            logits = plain.model_forward(w, cfg, toks)
+            for p in kept_positions(len(toks)):
+                want[(name, p)] = logits[p].numpy().copy()
+            del logits
+    del w
+    return d, reqs, want
+
+
+@pytest.fixture(scope="module", params=["float32", "bfloat16"])
+def engine_model(request, oracle):
+    from tensorline_amd.engine.loading import load_model
+    model, _ = load_model(oracle[0], request.param, "cuda:0")
+    yield request.param, model
+    del model
+    torch.cuda.empty_cache()
+
+
+def only_kept(steps, source_of=lambda rid: rid):
+    """The same steps, asking only for the logits at the kept positions of each request."""
+    done: dict[str, int] = {}
+    out = []
+    for st in steps:
+        entries = []
+        for e in st["entries"]:
+            base = done.get(e["id"], 0)
+            keep = set(kept_positions(LENGTHS[source_of(e["id"])]))
+            entries.append({"id": e["id"], "tokens": e["tokens"], "want": [w for w in e["want"] if base + w in keep]})
+            done[e["id"]] = base + len(e["tokens"])
+        out.append({"entries": entries, "end": st["end"]})
+    return out
+
+
+def compare(got, want, source_of=lambda rid: rid, limit=1e-5):
+    scale = {}
+    for (name, p), row in want.items():
+        scale[name] = max(scale.get(name, 0.0), float(np.abs(row).max()))
+    worst = 0.0
+    for (rid, p), row in got.items():
+        name = source_of(rid)
+        err = float(np.abs(row - want[(name, p)]).max()) / scale[name]
+        assert np.isfinite(err) and err < limit, f"request {rid} position {p}: relative error {err:.3e} >= {limit}"
+        worst = max(worst, err)
+    return worst
+
+
+CUTS = {"whole": helpers.steps_whole, "decode": helpers.steps_prefill_then_decode,
+        "portions": lambda reqs: helpers.steps_portions(reqs, sizes=(700, 130, 2, 64, 513, 17, 300, 3)),
+        "mixed": lambda reqs: helpers.steps_mixed(reqs, seed=3, tail=12)}
+
+
+@pytest.mark.parametrize("cut", list(CUTS))
+def test_cuttings_match_plain_at_real_layer_sizes(oracle, engine_model, cut):
+    from tensorline_amd.engine.replay import TraceSession
+    d, reqs, want = oracle
+    dtype, model = engine_model
+    steps = only_kept(CUTS[cut](reqs))
+    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=PAGE)
+    got = helpers.collect_logits(session.step, steps)
+    assert set(got) == set(want)
+    worst = compare(got, want, limit=LIMIT[dtype])
+    print(f"7B layer sizes, 2 layers, {cut} {dtype}: worst relative error {worst:.3e}")
+    assert session.cache.all_free()
+
+
+def batch_decode_steps(copies: dict[str, list[int]], tail: int, budget: int = 2048):
+    """Every request's tokens but the last ``tail`` as whole prompts, several to a step under a
+    token budget; then ``tail`` steps in which every request decodes one token."""
+    steps, entries, used = [], [], 0
+    for rid, toks in copies.items():
+        n = len(toks) - tail
+        if entries and used + n > budget:
+            steps.append({"entries": entries, "end": []})
+            entries, used = [], 0
+        entries.append({"id": rid, "tokens": toks[:n], "want": list(range(n))})
+        used += n
+    steps.append({"entries": entries, "end": []})
+    for i in range(tail, 0, -1):
+        steps.append({"entries": [{"id": rid, "tokens": [toks[len(toks) - i]], "want": [0]} for rid, toks in copies.items()],
+                      "end": list(copies) if i == 1 else []})
+    return steps
+
+
+@pytest.mark.parametrize("rows, graphs", [(8, False), (8, True), (40, False), (40, True)],
+                         ids=["8-rows-eager", "8-rows-graph", "40-rows-eager", "40-rows-graph"])
+def test_decoding_many_rows_at_real_layer_sizes(oracle, engine_model, rows, graphs):
+    """The last 32 tokens of 8 and of 40 requests decoded together: the few-row and the
+    17-to-64-row kernels of the bfloat16 path, eagerly and replayed from the graphs of the buckets
+    of 8 and of 40 rows."""
+    from tensorline_amd.engine.replay import TraceSession
+    d, reqs, want = oracle
+    dtype, model = engine_model
+    names = ["short", "mid", "long", "short", "mid"] if rows == 8 else ["short", "mid"]
+    source = {f"c{i}": ("long" if rows == 40 and i in (7, 31) else names[i % len(names)]) for i in range(rows)}
+    copies = {rid: reqs[name] for rid, name in source.items()}
+    steps = only_kept(batch_decode_steps(copies, tail=32), source.get)
+    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=PAGE, max_requests=rows, graphs=graphs)
+    got = helpers.collect_logits(session.step, steps)
+    assert {(source[rid], p) for rid, p in got} == {k for k in want if k[0] in set(source.values())}
+    worst = compare(got, want, source.get, LIMIT[dtype])
+    print(f"7B layer sizes, 2 layers, {rows} rows decoding, graphs={graphs}, {dtype}: worst relative error {worst:.3e}")
+    if graphs:
+        assert session.runner.graph_replays == 32
+        assert max(session.runner.graphs) >= rows and (rows <= 16 or max(session.runner.graphs) > 16)
+    assert session.cache.all_free()
