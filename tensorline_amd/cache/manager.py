@@ -1,8 +1,10 @@
 """The cache manager: paged keys and values per group of layers, page tables per request, and
 slots for fixed-size per-request state.
 
-* **Groups.**  Schedule entries whose mixers keep the same thing per token (same head count and
-  size, same window) form a group.  A group has its own page pool: its own page ids and one
+* **Groups.**  Schedule entries whose mixers keep the same thing per token (the same planes, see
+  :class:`tensorline_amd.parts.spec.CacheNeed`, and the same window) form a group.  What a plane
+  means (keys, values, something else) is the mixer's business: the manager allocates
+  ``[pages, page, *shape]`` or ``[pages, *shape, page]`` per plane and entry, and hands them out by name.  A group has its own page pool: its own page ids and one
   allocator; within a group one page id addresses the same page in every member's storage
   (reference: one id for all layers, tensorline/paged.py:128-130).  An entry that reads another
   entry's cache belongs to that entry's group and has no storage of its own.
@@ -32,13 +34,16 @@ from tensorline_amd.parts.spec import CacheNeed, ScheduleEntry, StateNeed
 _TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
 
 
+def _plane_dtype(name: str, compute: torch.dtype) -> torch.dtype:
+    return compute if name == "compute" else _TORCH_DTYPES[name]
+
+
 @dataclass
 class CacheGroup:
     need: CacheNeed
     entries: list[int]                       # schedule entries with storage in this group
     allocator: PagePool
-    k: dict[int, torch.Tensor] = field(default_factory=dict)
-    v: dict[int, torch.Tensor] = field(default_factory=dict)
+    storage: dict[int, dict[str, torch.Tensor]] = field(default_factory=dict)   # entry -> plane name -> pages
 
     @property
     def window(self) -> int:
@@ -77,8 +82,8 @@ class CacheManager:
             if e.cache_from is not None:
                 src = e.cache_from
                 src_need = cache_needs[src]
-                if src_need is None or (src_need.num_kv_heads, src_need.head_dim) != (need.num_kv_heads, need.head_dim):
-                    raise ValueError(f"schedule entry {i} reads the cache of entry {src}, whose keys have another shape")
+                if src_need is None or src_need.planes != need.planes:
+                    raise ValueError(f"schedule entry {i} reads the cache of entry {src}, which keeps something else per token")
                 self.group_of_entry[i] = self.group_of_entry[src]
                 self.storage_entry[i] = src
                 continue
@@ -114,12 +119,11 @@ class CacheManager:
 
         if allocate_storage:
             for g in self.groups:
-                # keys [pages, page, nkv, d]; values transposed within the page: [pages, nkv, d, page]
-                k_shape = (num_blocks + 1, page_size, g.need.num_kv_heads, g.need.head_dim)
-                v_shape = (num_blocks + 1, g.need.num_kv_heads, g.need.head_dim, page_size)
-                for i in g.entries:
-                    g.k[i] = torch.zeros(k_shape, dtype=dtype, device=device)
-                    g.v[i] = torch.zeros(v_shape, dtype=dtype, device=device)
+                for i in g.entries:                       # one page more than the pool: the scratch page
+                    g.storage[i] = {
+                        plane.name: torch.zeros(plane.storage_shape(num_blocks + 1, page_size),
+                                                dtype=_plane_dtype(plane.dtype, dtype), device=device)
+                        for plane in g.need.planes}
             for i, need in enumerate(self.state_needs):
                 if need is not None:
                     self.state[i] = torch.zeros((max_requests + 1, *need.shape), dtype=_TORCH_DTYPES[need.dtype], device=device)
@@ -130,12 +134,15 @@ class CacheManager:
     @staticmethod
     def bytes_per_page(cache_needs: Sequence[CacheNeed | None], schedule: Sequence[ScheduleEntry], page_size: int,
                        elem_size: int) -> int:
-        """Bytes one page id costs over all entries with storage (2 for keys and values; reference:
-        tensorline/paged.py:132-137)."""
+        """Bytes one page id costs over all entries with storage: every plane of every such entry
+        (keys and values of each layer in the reference: tensorline/paged.py:132-137).  ``elem_size``
+        is that of the cache's own dtype."""
         total = 0
         for e, need in zip(schedule, cache_needs):
             if need is not None and e.cache_from is None:
-                total += 2 * page_size * need.num_kv_heads * need.head_dim * elem_size
+                for plane in need.planes:
+                    size = elem_size if plane.dtype == "compute" else torch.empty(0, dtype=_TORCH_DTYPES[plane.dtype]).element_size()
+                    total += page_size * plane.values_per_token() * size
         return total
 
     def pages_for(self, tokens: int) -> int:
@@ -307,12 +314,13 @@ class CacheManager:
             alloc.publish(table[i], h, content)
 
     # ---- views for the step function -------------------------------------------------------
-    def storage(self, entry: int) -> tuple[torch.Tensor | None, torch.Tensor | None]:
+    def storage(self, entry: int) -> dict[str, torch.Tensor]:
+        """The pages of the entry's planes by name (those of the entry whose cache it reads, if it
+        has none of its own); empty for an entry that caches nothing."""
         src = self.storage_entry[entry]
         if src is None:
-            return None, None
-        g = self.groups[self.group_of_entry[entry]]
-        return g.k.get(src), g.v.get(src)
+            return {}
+        return self.groups[self.group_of_entry[entry]].storage.get(src, {})
 
     def owns_storage(self, entry: int) -> bool:
         return self.storage_entry[entry] == entry

@@ -45,12 +45,19 @@ class AttentionPlan:
 @dataclass
 class LayerCache:
     """The cache as one schedule entry sees it in this step."""
-    k: torch.Tensor | None
-    v: torch.Tensor | None
+    planes: dict[str, torch.Tensor]   # the pages of each plane its mixer declared, by name
     slots: torch.Tensor | None        # int32 [T]: cache row of each token of the step
     tables: torch.Tensor | None       # int32 [S, NB]: page ids of each sequence
     write: bool                       # False: the entry reads a cache another entry wrote
     state: torch.Tensor | None = None  # [slots + 1, *shape] fixed-size per-request state, if any
+
+    @property
+    def k(self) -> torch.Tensor | None:
+        return self.planes.get("k")
+
+    @property
+    def v(self) -> torch.Tensor | None:
+        return self.planes.get("v")
 
 
 @dataclass

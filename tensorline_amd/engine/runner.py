@@ -71,9 +71,8 @@ class ModelRunner:
         views: list[LayerCache] = []
         for i in range(len(self.model.schedule)):
             g = cache.group_of_entry[i]
-            k, v = cache.storage(i)
             views.append(LayerCache(
-                k=k, v=v, slots=g_slots[g] if g is not None else None,
+                planes=cache.storage(i), slots=g_slots[g] if g is not None else None,
                 tables=g_tables[g] if g is not None else None,
                 write=cache.owns_storage(i), state=cache.state.get(i)))
         return ctx, views

@@ -12,9 +12,8 @@ from typing import Callable
 import torch
 
 from tensorline_amd.ops import kernels
-from tensorline_amd.parts.base import Linear
 from tensorline_amd.parts.registry import BLOCKS, build_part, _ensure_builtin
-from tensorline_amd.parts.spec import CacheNeed, ModelSpec, StateNeed, TensorDecl
+from tensorline_amd.parts.spec import CacheNeed, Intake, ModelSpec, StateNeed, TensorDecl
 
 
 class DecoderModel:
@@ -25,6 +24,8 @@ class DecoderModel:
         self.dtype = dtype
         self.device = device
         self.hidden_size, self.vocab_size = spec.hidden_size, spec.vocab_size
+        common = dict(hidden_size=spec.hidden_size, dtype=dtype, device=device)
+        self.embedding = build_part("embedding", spec.embedding, layer_prefix="", vocab_size=spec.vocab_size, **common)
         self.blocks = []
         for layer in spec.layers:
             try:
@@ -33,115 +34,104 @@ class DecoderModel:
                 raise ValueError(f"unknown block kind {layer.block!r}; known: {', '.join(sorted(BLOCKS))}") from None
             self.blocks.append(cls(layer, spec.hidden_size, dtype, device))
         self.schedule = spec.run_order()
-        self.final_norm = build_part("norm", spec.final_norm, layer_prefix="", hidden_size=spec.hidden_size,
-                                     dtype=dtype, device=device)
-        self.embed_name = spec.embedding.params["name"]
-        self.head_name = spec.head.params["name"]
-        self.tied = bool(spec.head.params.get("tied", False))
-        self.embed_table: torch.Tensor | None = None
-        self.head = Linear(self.head_name.removesuffix(".weight"), spec.hidden_size, spec.vocab_size, False)
+        self.final_norm = build_part("norm", spec.final_norm, layer_prefix="", **common)
+        self.head = build_part("head", spec.head, layer_prefix="", vocab_size=spec.vocab_size, **common)
+        self._after: list[Intake | None] | None = None     # per schedule entry: what its successor takes
+
+    def _all_parts(self):
+        yield self.embedding
+        for b in self.blocks:
+            yield from b.parts()
+        yield self.final_norm
+        yield self.head
 
     # ---- weights -----------------------------------------------------------------------
     def tensor_decls(self) -> dict[str, TensorDecl]:
-        H, V = self.hidden_size, self.vocab_size
-        out: dict[str, TensorDecl] = {self.embed_name: TensorDecl((V, H), "normal", 0.02, "compute")}
-        for b in self.blocks:
-            for p in b.parts():
-                out.update(p.tensors())
-        out.update(self.final_norm.tensors())
-        if not self.tied:
-            out[self.head_name] = TensorDecl((V, H), "normal", 0.02, "compute")
+        out: dict[str, TensorDecl] = {}
+        for p in self._all_parts():
+            out.update(p.tensors())
         return out
 
     def optional_tensors(self) -> dict[str, str]:
         """Names a checkpoint may also hold, with the declared tensor each must then equal."""
-        return {self.head_name: self.embed_name} if self.tied else {}
+        fn = getattr(self.head, "optional_tensors", None)
+        return fn(self.embedding) if fn is not None else {}
 
     def load_tensors(self, get: Callable[[str], torch.Tensor]) -> None:
-        self.embed_table = get(self.embed_name)
+        self.embedding.load(get)
         for b in self.blocks:
             for p in b.parts():
                 p.load(get)
         self.final_norm.load(get)
-        self.head.weight = self.embed_table if self.tied else get(self.head_name)
-        self.head.prepare()
+        self.head.load(get, self.embedding)
+        self._after = None
 
     def weight_bytes(self) -> int:
         """Bytes of weights on the device, a shared tensor counted once (reference: quant.py:107-113)."""
         seen, total = set(), 0
-        tensors = [self.embed_table] + self.head.tensors_kept() + self.final_norm.weight_tensors()
-        for b in self.blocks:
-            for p in b.parts():
-                tensors += p.weight_tensors()
-        for t in tensors:
-            if t is None or t.data_ptr() in seen:
-                continue
-            seen.add(t.data_ptr())
-            total += t.numel() * t.element_size()
+        for p in self._all_parts():
+            for t in p.weight_tensors():
+                if t is None or t.data_ptr() in seen:
+                    continue
+                seen.add(t.data_ptr())
+                total += t.numel() * t.element_size()
         return total
 
     # ---- what the cache manager has to provide ------------------------------------------
     def cache_needs(self) -> list[CacheNeed | None]:
-        """Per schedule entry: the keys/values its mixer keeps per token, or None."""
-        out = []
-        for e in self.schedule:
-            mixer = self.blocks[e.layer].mixer
-            need = mixer.cache_need() if hasattr(mixer, "cache_need") else None
-            out.append(need)
-        return out
+        """Per schedule entry: what its block keeps per cached token, or None."""
+        return [self.blocks[e.layer].cache_need() for e in self.schedule]
 
     def state_needs(self) -> list[StateNeed | None]:
-        """Per schedule entry: the fixed-size per-request state its mixer keeps, or None."""
-        out = []
-        for e in self.schedule:
-            mixer = self.blocks[e.layer].mixer
-            out.append(mixer.state_need() if hasattr(mixer, "state_need") else None)
-        return out
+        """Per schedule entry: the fixed-size per-request state its block keeps, or None."""
+        return [self.blocks[e.layer].state_need() for e in self.schedule]
 
     # ---- one step ------------------------------------------------------------------------
     def tune_library(self, rows: int) -> int:
         """Let the library choose its kernels by measurement for steps of ``rows`` tokens (a full
         prompt portion): one search per distinct product shape.  Returns how many were searched."""
         seen, done = set(), 0
-        for block in self.blocks:
-            for part in block.parts():
-                for weight, out_dtype in getattr(part, "library_products", lambda: [])():
-                    key = (tuple(weight.shape), weight.dtype, out_dtype)
-                    if key in seen:
-                        continue
-                    seen.add(key)
-                    done += bool(kernels.tune_library_linear(rows, weight, out_dtype))
+        for part in self._all_parts():
+            for weight, out_dtype in getattr(part, "library_products", lambda: [])():
+                key = (tuple(weight.shape), weight.dtype, out_dtype)
+                if key in seen:
+                    continue
+                seen.add(key)
+                done += bool(kernels.tune_library_linear(rows, weight, out_dtype))
         return done
+
+    def _tail_intake(self) -> Intake:
+        """What the final norm and the head take from the last block."""
+        carried = None
+        if getattr(self.head, "takes_normed_rows", lambda: False)():
+            fn = getattr(self.final_norm, "deferrable", None)
+            carried = fn() if fn is not None else None
+        return Intake(carried, bool(getattr(self.final_norm, "adds_share_sums", False)))
+
+    def _negotiate(self) -> list[Intake | None]:
+        """For every schedule entry the intake of whoever runs after it, or None for a block that
+        takes no ``after=`` (then it returns a tensor, which everybody takes)."""
+        takers = [self.blocks[e.layer] for e in self.schedule]
+        intakes = [b.intake() if hasattr(b, "intake") else Intake() for b in takers[1:]] + [self._tail_intake()]
+        return [nxt if hasattr(b, "intake") else None for b, nxt in zip(takers, intakes)]
 
     def forward(self, ctx, caches) -> torch.Tensor:
         """``caches[i]`` is the view of the cache for schedule entry ``i``."""
-        x = kernels.embed(ctx.ids, self.embed_table)
-        pending = None
-        last = len(self.schedule) - 1
+        if self._after is None:
+            self._after = self._negotiate()
+        x = self.embedding.forward(ctx.ids)
+        carry = None
         for i, e in enumerate(self.schedule):
-            block = self.blocks[e.layer]
-            if getattr(block, "takes_normed_rows", None) is None:
-                pending = block.forward(x, pending, ctx, caches[i])      # a block that knows no hand-off
-                continue
-            # the norm after this block: as next_norm if whoever applies it can take it as
-            # NormedRows, as pending_norm if it adds a product left in its K shares
-            next_norm = after = None
-            if i < last:
-                nxt = self.blocks[self.schedule[i + 1].layer]
-                after = getattr(nxt, "mixer_norm", None)
-                if getattr(nxt, "takes_normed_rows", lambda: False)():
-                    next_norm = nxt.mixer_norm
+            block, after = self.blocks[e.layer], self._after[i]
+            if after is None:
+                carry = block.forward(x, carry, ctx, caches[i])
             else:
-                after = self.final_norm
-                if self.head.shuffled is not None:
-                    next_norm = self.final_norm
-            pending_norm = after if getattr(after, "adds_share_sums", False) else None
-            pending = block.forward(x, pending, ctx, caches[i], next_norm=next_norm, pending_norm=pending_norm)
+                carry = block.forward(x, carry, ctx, caches[i], after=after)
         if ctx.logit_rows.numel() == 0:
             # the residual stream is complete only after the last add; nothing reads it here
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=x.device)
-        if isinstance(pending, kernels.NormedRows):
-            h = pending if ctx.logits_for_all_rows else pending.take(ctx.logit_rows)
+        if isinstance(carry, kernels.NormedRows):
+            h = carry if ctx.logits_for_all_rows else carry.take(ctx.logit_rows)
         else:
-            h = self.final_norm.forward(x, pending, rows=ctx.logit_rows)
-        return self.head(h, out_dtype=torch.float32)
+            h = self.final_norm.forward(x, carry, rows=ctx.logit_rows)
+        return self.head.forward(h)

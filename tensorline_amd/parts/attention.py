@@ -13,7 +13,7 @@ import torch
 from tensorline_amd.ops import kernels
 from tensorline_amd.parts.base import Linear, Part, TensorGetter, fuse_linears
 from tensorline_amd.parts.registry import build_part, register_mixer
-from tensorline_amd.parts.spec import CacheNeed, PartSpec
+from tensorline_amd.parts.spec import CacheNeed, PartSpec, keys_and_values
 
 
 @register_mixer("attention")
@@ -63,7 +63,7 @@ class PagedAttention(Part):
 
     # ---- what it keeps -------------------------------------------------------------------
     def cache_need(self) -> CacheNeed | None:
-        return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
+        return keys_and_values(self.num_kv_heads, self.head_dim, self.window)
 
     def state_need(self):
         return None

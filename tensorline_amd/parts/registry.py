@@ -14,8 +14,11 @@ FEED_FORWARDS: dict[str, type] = {}
 NORMS: dict[str, type] = {}
 POSITIONS: dict[str, type] = {}
 BLOCKS: dict[str, type] = {}
+EMBEDDINGS: dict[str, type] = {}
+HEADS: dict[str, type] = {}
 
-_TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "position": POSITIONS, "block": BLOCKS}
+_TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "position": POSITIONS, "block": BLOCKS,
+           "embedding": EMBEDDINGS, "head": HEADS}
 
 
 def _register(table: dict[str, type], what: str, kind: str, replace: bool) -> Callable[[type], type]:
@@ -47,6 +50,14 @@ def register_block(kind: str, replace: bool = False):
     return _register(BLOCKS, "block", kind, replace)
 
 
+def register_embedding(kind: str, replace: bool = False):
+    return _register(EMBEDDINGS, "embedding", kind, replace)
+
+
+def register_head(kind: str, replace: bool = False):
+    return _register(HEADS, "head", kind, replace)
+
+
 def build_part(what: str, spec: PartSpec, layer_prefix: str | None = None, **common):
     """Instantiate the part ``spec`` names: ``cls(**common, **spec.params)``; parts that read
     checkpoint tensors get ``prefix = layer_prefix + spec.prefix``."""
@@ -64,6 +75,7 @@ def build_part(what: str, spec: PartSpec, layer_prefix: str | None = None, **com
 def _ensure_builtin() -> None:
     import tensorline_amd.parts.attention  # noqa: F401
     import tensorline_amd.parts.block  # noqa: F401
+    import tensorline_amd.parts.embedding  # noqa: F401
     import tensorline_amd.parts.feedforward  # noqa: F401
     import tensorline_amd.parts.norm  # noqa: F401
     import tensorline_amd.parts.rotary  # noqa: F401

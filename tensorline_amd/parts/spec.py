@@ -57,6 +57,17 @@ class ScheduleEntry:
 
 
 @dataclass(frozen=True)
+class Intake:
+    """What whoever runs after a block can take in place of a plain pending tensor; a block is
+    told the intake of its successor and may answer with the cheaper form.
+    ``normed_rows_for``: (weight, eps) of the norm the successor applies first, if it takes that
+    norm's input as ``tensorline_amd.ops.kernels.NormedRows``.  ``share_sums``: its first norm adds a
+    product left in its shares of K (``tensorline_amd.ops.kernels.ShareSum``)."""
+    normed_rows_for: tuple | None = None
+    share_sums: bool = False
+
+
+@dataclass(frozen=True)
 class ModelSpec:
     hidden_size: int
     vocab_size: int
@@ -86,16 +97,54 @@ class ModelSpec:
 
 
 @dataclass(frozen=True)
+class CachePlane:
+    """One tensor a mixer keeps for every cached token: ``shape`` per token, in the cache's dtype
+    (``dtype`` "compute") or a fixed one.  The cache manager lays it out in pages and knows nothing
+    else about it: ``token_axis`` "first" gives storage ``[pages, page, *shape]`` (a token's values
+    contiguous), "last" gives ``[pages, *shape, page]`` (a page's tokens contiguous innermost)."""
+    name: str
+    shape: tuple[int, ...]
+    token_axis: str = "first"
+    dtype: str = "compute"
+
+    def __post_init__(self):
+        if self.token_axis not in ("first", "last"):
+            raise ValueError(f"cache plane {self.name!r}: token_axis must be 'first' or 'last'")
+        if not self.shape or min(self.shape) <= 0:
+            raise ValueError(f"cache plane {self.name!r}: a token's shape must be non-empty and positive")
+
+    def storage_shape(self, pages: int, page_size: int) -> tuple[int, ...]:
+        return (pages, page_size, *self.shape) if self.token_axis == "first" else (pages, *self.shape, page_size)
+
+    def values_per_token(self) -> int:
+        n = 1
+        for d in self.shape:
+            n *= d
+        return n
+
+
+@dataclass(frozen=True)
 class CacheNeed:
-    """What a mixer keeps per token: keys and values of ``num_kv_heads`` x ``head_dim``, for all
-    earlier tokens (``window`` 0) or for the last ``window`` of them."""
-    num_kv_heads: int
-    head_dim: int
+    """What a mixer keeps per token: one or more planes, for all earlier tokens (``window`` 0) or
+    for the last ``window`` of them.  Mixers with equal needs share a pool of pages."""
+    planes: tuple[CachePlane, ...]
     window: int = 0
+
+    def __post_init__(self):
+        names = [p.name for p in self.planes]
+        if not names or len(set(names)) != len(names):
+            raise ValueError("a cache need has at least one plane, each with a name of its own")
 
     @property
     def kind(self) -> str:
         return "window" if self.window > 0 else "full"
+
+
+def keys_and_values(num_kv_heads: int, head_dim: int, window: int = 0) -> CacheNeed:
+    """The need of an attention mixer: keys ``k`` stored token by token, values ``v`` stored with
+    the tokens of a page innermost (what the attention kernels read in one piece each)."""
+    per_token = (int(num_kv_heads), int(head_dim))
+    return CacheNeed((CachePlane("k", per_token, "first"), CachePlane("v", per_token, "last")), int(window))
 
 
 @dataclass(frozen=True)

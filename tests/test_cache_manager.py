@@ -8,7 +8,7 @@ from hypothesis import given, settings, strategies as st
 
 from tensorline_amd.cache.allocator import PagePool, page_key
 from tensorline_amd.cache.manager import CacheManager
-from tensorline_amd.parts.spec import CacheNeed, ScheduleEntry, StateNeed
+from tensorline_amd.parts.spec import keys_and_values, ScheduleEntry, StateNeed
 
 
 def test_allocator_refcount_lru_and_eviction():
@@ -100,13 +100,13 @@ def manager(needs, schedule=None, states=None, **kw):
 
 
 def test_groups_tables_and_storage():
-    full, win = CacheNeed(2, 8), CacheNeed(2, 8, window=6)
+    full, win = keys_and_values(2, 8), keys_and_values(2, 8, window=6)
     m = manager([full, win, full, None], states=[None, None, None, StateNeed((5,))])
     assert len(m.groups) == 2 and m.group_of_entry == [0, 1, 0, None]
     assert m.groups[0].entries == [0, 2] and m.groups[1].entries == [1]
-    k, v = m.storage(2)
+    k, v = m.storage(2)["k"], m.storage(2)["v"]
     assert tuple(k.shape) == (17, 4, 2, 8) and tuple(v.shape) == (17, 2, 8, 4)     # one scratch page; V transposed
-    assert m.storage(3) == (None, None) and tuple(m.state[3].shape) == (5, 5)
+    assert m.storage(3) == {} and tuple(m.state[3].shape) == (5, 5)
     per_page = CacheManager.bytes_per_page([full, win, full, None], [ScheduleEntry(i) for i in range(4)], 4, 2)
     assert per_page == 3 * 2 * 4 * 2 * 8 * 2
     assert m.add_request("a") is not None
@@ -119,7 +119,7 @@ def test_groups_tables_and_storage():
 
 
 def test_window_pages_are_given_back_and_used_again():
-    m = manager([CacheNeed(1, 8), CacheNeed(1, 8, window=6)], num_blocks=6)
+    m = manager([keys_and_values(1, 8), keys_and_values(1, 8, window=6)], num_blocks=6)
     m.add_request("a")
     computed = 0
     for n in (5, 4, 3, 7, 1, 1, 1):
@@ -134,19 +134,19 @@ def test_window_pages_are_given_back_and_used_again():
         assert all(b >= 0 for b in m.table("a", 0))                                 # the full group keeps everything
     assert computed == 22 and len(m.table("a", 0)) == 6
     assert m.num_free(1) >= 3            # 22 tokens in 6 pages of 4: the windowed group never holds more than 3 at rest
-    assert m.can_ever_hold(200, step_tokens=4) is False and manager([CacheNeed(1, 8, window=6)], num_blocks=6).can_ever_hold(200, 4)
+    assert m.can_ever_hold(200, step_tokens=4) is False and manager([keys_and_values(1, 8, window=6)], num_blocks=6).can_ever_hold(200, 4)
     m.release("a")
     assert m.all_free()
 
 
 def test_shared_cache_entry_and_bad_schedules():
-    need = CacheNeed(2, 8)
+    need = keys_and_values(2, 8)
     m = manager([need, need], schedule=[ScheduleEntry(0), ScheduleEntry(0, cache_from=0)])
-    assert m.group_of_entry == [0, 0] and m.storage(1)[0] is m.storage(0)[0] and not m.owns_storage(1)
-    with pytest.raises(ValueError, match="another shape"):
-        manager([need, CacheNeed(1, 8)], schedule=[ScheduleEntry(0), ScheduleEntry(0, cache_from=0)])
+    assert m.group_of_entry == [0, 0] and m.storage(1)["k"] is m.storage(0)["k"] and not m.owns_storage(1)
+    with pytest.raises(ValueError, match="something else per token"):
+        manager([need, keys_and_values(1, 8)], schedule=[ScheduleEntry(0), ScheduleEntry(0, cache_from=0)])
     with pytest.raises(ValueError, match="further back"):
-        manager([CacheNeed(2, 8, window=4), need], schedule=[ScheduleEntry(0), ScheduleEntry(0, cache_from=0)])
+        manager([keys_and_values(2, 8, window=4), need], schedule=[ScheduleEntry(0), ScheduleEntry(0, cache_from=0)])
 
 
 def test_state_slots():
@@ -162,7 +162,7 @@ def test_state_slots():
 
 
 def test_prefix_sharing_through_the_manager():
-    m = manager([CacheNeed(1, 8)], prefix_caching=True)
+    m = manager([keys_and_values(1, 8)], prefix_caching=True)
     toks = list(range(11))
     m.add_request("a")
     assert m.match_prefix("a", toks) == 0 and m.grow("a", 11)
@@ -179,15 +179,15 @@ def test_prefix_sharing_through_the_manager():
     assert m.match_prefix("d", toks) == 8
     m.release("d")
     # windows or state switch it off
-    assert not manager([CacheNeed(1, 8, window=4)], prefix_caching=True).prefix_caching
-    assert not manager([CacheNeed(1, 8), None], states=[None, StateNeed((2,))], prefix_caching=True).prefix_caching
+    assert not manager([keys_and_values(1, 8, window=4)], prefix_caching=True).prefix_caching
+    assert not manager([keys_and_values(1, 8), None], states=[None, StateNeed((2,))], prefix_caching=True).prefix_caching
 
 
 @settings(max_examples=60, deadline=None)
 @given(seed=st.integers(0, 10 ** 6), window=st.sampled_from([0, 5, 9]), prefix=st.booleans())
 def test_random_orders_keep_every_page_accounted_for(seed, window, prefix):
     rng = random.Random(seed)
-    needs = [CacheNeed(1, 8), CacheNeed(1, 8, window=window)] if window else [CacheNeed(1, 8)]
+    needs = [keys_and_values(1, 8), keys_and_values(1, 8, window=window)] if window else [keys_and_values(1, 8)]
     m = manager(needs, num_blocks=12, max_requests=3, prefix_caching=prefix, allocate_storage=False)
     live: dict[int, int] = {}
     toks = {}
@@ -220,3 +220,27 @@ def test_random_orders_keep_every_page_accounted_for(seed, window, prefix):
         m.release(rid)
     m.check()
     assert m.all_free()
+
+
+def test_a_mixer_may_declare_any_planes_and_the_manager_only_lays_them_out():
+    """Not keys and values: one compressed vector per token kept in the cache's dtype and a float32
+    score per token and head, the latter with a page's tokens innermost.  The manager allocates what
+    is declared, counts its bytes, and groups entries by equal declarations."""
+    from tensorline_amd.parts.spec import CacheNeed, CachePlane
+    latent = CacheNeed((CachePlane("latent", (24,)), CachePlane("gate", (3,), token_axis="last", dtype="float32")))
+    kv = keys_and_values(2, 8)
+    m = manager([latent, kv, latent], dtype=torch.bfloat16, page_size=4, num_blocks=5)
+    assert m.group_of_entry == [0, 1, 0] and len(m.groups) == 2
+    planes = m.storage(2)
+    assert set(planes) == {"latent", "gate"} and planes["latent"] is not m.storage(0)["latent"]
+    assert tuple(planes["latent"].shape) == (6, 4, 24) and planes["latent"].dtype == torch.bfloat16
+    assert tuple(planes["gate"].shape) == (6, 3, 4) and planes["gate"].dtype == torch.float32
+    assert set(m.storage(1)) == {"k", "v"}
+    sched = [ScheduleEntry(i) for i in range(3)]
+    assert CacheManager.bytes_per_page([latent, kv, latent], sched, 4, 2) == 2 * 4 * (24 * 2 + 3 * 4) + 4 * 2 * (2 * 8) * 2
+    with pytest.raises(ValueError):
+        CacheNeed(())
+    with pytest.raises(ValueError):
+        CacheNeed((CachePlane("a", (2,)), CachePlane("a", (3,))))
+    with pytest.raises(ValueError):
+        CachePlane("a", (2,), token_axis="middle")

@@ -83,7 +83,7 @@ def test_random_model_round_trip(folder):
     attn = model.blocks[1].mixer
     want = torch.cat([raw[f"model.layers.1.self_attn.{n}_proj.weight"] for n in "qkv"]).float()
     assert torch.equal(attn.qkv.weight, want) and attn.qkv.weight.dtype == torch.float32
-    assert torch.equal(model.head.weight, raw["lm_head.weight"].float())
+    assert torch.equal(model.head.linear.weight, raw["lm_head.weight"].float())
     assert torch.equal(model.final_norm.weight, raw["model.norm.weight"].float())
     # the same seed gives the same model, another seed another
     d2 = write_random_model(cfg, d + "2", seed=3)
@@ -100,7 +100,7 @@ def test_storage_dtypes(folder):
     d, _ = folder
     model, _ = load_model(d, "bfloat16", "cpu")
     attn = model.blocks[0].mixer
-    assert attn.qkv.weight.dtype == torch.bfloat16 and model.embed_table.dtype == torch.bfloat16
+    assert attn.qkv.weight.dtype == torch.bfloat16 and model.embedding.table.dtype == torch.bfloat16
     assert attn.qkv.bias.dtype == torch.float32 and model.final_norm.weight.dtype == torch.float32
     assert attn.qkv.shuffled is not None and attn.qkv.shuffled.shape[-3:] == (4, 16, 8)
     # a tensor stored in 32-bit that the model keeps in 32-bit stays exact
@@ -140,7 +140,7 @@ def test_wrong_dtypes_are_an_error_and_extra_tensors_alone_a_warning(folder):
     save_file(raw, path)
     with pytest.warns(UserWarning, match="rotary.inv_freq"):
         model, _ = load_model(d, "float32", "cpu")
-    assert torch.equal(model.embed_table, good["model.embed_tokens.weight"].float())
+    assert torch.equal(model.embedding.table, good["model.embed_tokens.weight"].float())
     # integer and 64-bit tensors under the names of float weights: one error names each, and the extra tensor too
     raw["model.layers.1.mlp.down_proj.weight"] = torch.zeros_like(good["model.layers.1.mlp.down_proj.weight"], dtype=torch.int64)
     raw["model.norm.weight"] = good["model.norm.weight"].double()
@@ -168,8 +168,8 @@ def test_tied_head(tmp_path):
     raw = load_file(path)
     assert "lm_head.weight" not in raw
     model, _ = load_model(d, "float32", "cpu")
-    assert model.head.weight is model.embed_table                           # shared, not copied
-    one = sum(t.numel() * t.element_size() for t in [model.embed_table])
+    assert model.head.linear.weight is model.embedding.table                           # shared, not copied
+    one = sum(t.numel() * t.element_size() for t in [model.embedding.table])
     assert model.weight_bytes() < 2 * one + 10 ** 6
     raw["lm_head.weight"] = raw["model.embed_tokens.weight"].clone()         # stored too, and equal: accepted
     save_file(raw, path)
@@ -201,7 +201,7 @@ def test_sharded_checkpoint(folder):
         json.dump({"weight_map": {**{n: "model-00001-of-00002.safetensors" for n in a},
                                   **{n: "model-00002-of-00002.safetensors" for n in b}}}, f)
     model, _ = load_model(d, "float32", "cpu")
-    assert torch.equal(model.embed_table, raw["model.embed_tokens.weight"].float())
+    assert torch.equal(model.embedding.table, raw["model.embed_tokens.weight"].float())
 
 
 def test_engine_refuses_to_run_without_a_gpu(folder):

@@ -131,7 +131,7 @@ def test_graph_decode_matches_eager_and_isolates_padding(folder_b):
         for i, s in enumerate(seqs):
             assert c.grow(i, len(s) + 21)
         assert all(bystander not in c.table(i) for i in range(3))
-        c.groups[0].k[0][bystander].fill_(7.0)
+        c.storage(0)["k"][bystander].fill_(7.0)
     first = [StepEntry(i, s, 0, [len(s) - 1]) for i, s in enumerate(seqs)]
     le, lg = eager.step(first), graph.step(first)      # not pure decode: both run eagerly
     torch.testing.assert_close(le, lg, atol=0, rtol=0)
@@ -145,7 +145,7 @@ def test_graph_decode_matches_eager_and_isolates_padding(folder_b):
         assert lg.argmax(-1).tolist() == le.argmax(-1).tolist(), step
         torch.testing.assert_close(lg, le, atol=1e-5, rtol=1e-5)
     assert graph.graph_replays == 20 and len(graph.graphs) == 1
-    assert torch.all(cg.groups[0].k[0][bystander] == 7.0)
+    assert torch.all(cg.storage(0)["k"][bystander] == 7.0)
 
 
 def test_parts_alone(folder_b):

@@ -7,7 +7,7 @@ import torch
 from tensorline_amd.cache.manager import CacheManager
 from tensorline_amd.engine.batch import StepEntry
 from tensorline_amd.engine.graphs import GraphRunner, _Captured
-from tensorline_amd.parts.spec import CacheNeed, ScheduleEntry
+from tensorline_amd.parts.spec import keys_and_values, ScheduleEntry
 
 
 class _Model:
@@ -17,7 +17,7 @@ class _Model:
 
 
 def _setup(window=0, page=4, max_blocks=8):
-    cache = CacheManager([CacheNeed(1, 8, window)], [ScheduleEntry(0)], [None], page_size=page, num_blocks=40,
+    cache = CacheManager([keys_and_values(1, 8, window)], [ScheduleEntry(0)], [None], page_size=page, num_blocks=40,
                          max_requests=4, dtype=torch.float32, device="cpu", allocate_storage=False)
     runner = GraphRunner(_Model(), cache, max_batch=4, max_blocks_per_seq=max_blocks)
     return cache, runner

@@ -8,7 +8,7 @@ from tensorline_amd.cache.manager import CacheManager
 from tensorline_amd.engine.engine import InferenceEngine
 from tensorline_amd.engine.loading import load_model
 from tensorline_amd.engine.scheduler import Request, RequestError, Scheduler
-from tensorline_amd.parts.spec import CacheNeed, ScheduleEntry
+from tensorline_amd.parts.spec import keys_and_values, ScheduleEntry
 from tensorline_amd.sampling.params import GenStats, SamplingParams
 from tests import helpers, plain
 
@@ -146,7 +146,7 @@ def test_temperature_sampling_is_seeded_and_batch_independent(tiny, cpu_kernels)
 
 # ---- decisions on host data only -----------------------------------------------------------------
 def host_cache(num_blocks, page=4, slots=8, window=0):
-    return CacheManager([CacheNeed(1, 8, window)], [ScheduleEntry(0)], [None], page_size=page, num_blocks=num_blocks,
+    return CacheManager([keys_and_values(1, 8, window)], [ScheduleEntry(0)], [None], page_size=page, num_blocks=num_blocks,
                         max_requests=slots, dtype=torch.float32, device="cpu", allocate_storage=False)
 
 
