@@ -145,3 +145,44 @@ def plain_logits(weights, cfg, reqs):
         for i in range(len(toks)):
             out[(rid, i)] = lg[i].to(torch.float32).numpy()
     return out
+
+
+# ---- looking into the engine from a test -------------------------------------------------------
+class ForcedSampler:
+    """Stands in for the engine's sampler: whatever the logits say, a request continues with the
+    tokens given for it (a request is known by its seed), and the logits it was shown are kept.
+    With the plain implementation's own tokens forced, a bfloat16 run sees the contexts the
+    plain run saw at every position, so its logits can be compared one by one; a token picked
+    from near-equal logits cannot send the rest of the comparison elsewhere."""
+
+    def __init__(self, forced: dict[int, list[int]]):
+        self.forced = forced
+        self.logits: dict[tuple[int, int], np.ndarray] = {}       # (seed, index of the generated token) -> row
+
+    def sample(self, logits, temperatures, top_ps, seeds, indices):
+        rows = logits.to(torch.float32).cpu().numpy()
+        out = []
+        for row, seed, index in zip(rows, seeds, indices):
+            self.logits[(seed, index)] = row.copy()
+            out.append(self.forced[seed][index])
+        return out
+
+
+def watch_pages(cache) -> dict:
+    """Count how often each page of each group is handed out from now on; ``reused(counts)`` then
+    says how many pages went to a second holder after the first gave them back."""
+    counts: dict[tuple[int, int], int] = {}
+    for gi, g in enumerate(cache.groups):
+        take = g.allocator.take
+
+        def counting(n, _take=take, _gi=gi):
+            got = _take(n)
+            for p in got or []:
+                counts[(_gi, p)] = counts.get((_gi, p), 0) + 1
+            return got
+        g.allocator.take = counting
+    return counts
+
+
+def reused(counts: dict) -> int:
+    return sum(1 for c in counts.values() if c > 1)

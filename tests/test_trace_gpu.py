@@ -53,11 +53,31 @@ def test_cuttings_match_plain(setup, cut, dtype):
     model, _ = load_model(d, dtype, "cuda:0")
     # the pool is as small as the trace allows, so pages are used again
     session = TraceSession(model, helpers.max_live_tokens(steps), page_size=helpers.PAGE[name])
+    pages = helpers.watch_pages(session.cache)
     got = helpers.collect_logits(session.step, steps)
     worst = _compare(got, want, reqs, LIMIT[dtype])
-    print(f"config {name} {cut} {dtype}: worst relative error {worst:.3e}")
+    print(f"config {name} {cut} {dtype}: worst relative error {worst:.3e}, {helpers.reused(pages)} pages used again")
     assert session.cache.all_free()
     session.cache.check()
+    if cut == "mixed":             # the point of the small pool: later requests compute on pages earlier ones left
+        assert helpers.reused(pages) >= 4, "no page was handed out twice: the pool is too large to test reuse"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_tail_replayed_from_graphs_matches_plain(setup, dtype):
+    """The cut that decodes the last 32 tokens one by one, with every pure decode step replayed
+    from a HIP graph as in serving (prompt portions still run eagerly): same logits."""
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.replay import TraceSession
+    name, d, reqs, want = setup
+    steps = helpers.steps_prefill_then_decode(reqs)
+    model, _ = load_model(d, dtype, "cuda:0")
+    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=helpers.PAGE[name], max_requests=4, graphs=True)
+    got = helpers.collect_logits(session.step, steps)
+    _compare(got, want, reqs, LIMIT[dtype])
+    # every token after a request's first step is a decode step, and every decode step replays
+    assert session.runner.graph_replays == sum(len(t) - max(1, len(t) - 32) for t in reqs.values())
+    assert session.cache.all_free()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
