@@ -7,9 +7,14 @@ A step is one decode step of the whole batch through the engine loop (schedule, 
 of the model, sampling, accept).  Weights are random (generated on the GPU from a seed), prompts
 are token ids uniform over the vocabulary.  One JSON line is printed: decoded tokens per second
 at the default batch, the prefill of one 2,048-token prompt, the decode step's share of the HBM
-roofline, and decode throughput at batch 1 and 64.  The fractions are of the published peaks;
-``machine`` holds what this GPU reaches on a plain copy and on a large library product, and the
-``frac_of_measured_*`` fields are the same figures relative to those.
+roofline, and under ``points`` decode throughput at batch 1 and 64 at the same context
+(``decode_b*``) and the decode phase of the workload the shape is quoted with, 2,048-token
+prompts and 256 generated tokens each, at batch 1, 8 and 64 (``gen_b*``), each with its time per
+step, its mean context and its share of the HBM roofline.  ``fp32`` holds the cost of the true
+32-bit path at the same layer sizes with fewer layers (both numbers are named).  The fractions
+are of the published peaks; ``machine`` holds what this GPU reaches on a plain copy and on a
+large library product, and the ``frac_of_measured_*`` fields are the same figures relative to
+those.  ``--profile`` adds the time of one eagerly run decode step by class of kernel.
 """
 from __future__ import annotations
 
@@ -105,11 +110,15 @@ def bench_decode(llm, batch: int, context: int, steps: int, warmup: int, seed: i
         eng.step()
     sync()
     assert all(not r.done for r in reqs) and len(eng.scheduler.running) == batch and not eng.scheduler.waiting
+    import torch
     c0 = eng.counters()
     lens0 = [len(r.tokens) for r in reqs]
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    e0.record()
     for _ in range(steps):
         eng.step()
+    e1.record()
     sync()
     dt = time.perf_counter() - t0
     c1 = eng.counters()
@@ -119,11 +128,74 @@ def bench_decode(llm, batch: int, context: int, steps: int, warmup: int, seed: i
     assert c1["preemptions"] == c0["preemptions"], "a sequence was preempted inside the timed steps"
     mean_ctx = (sum(lens0) + sum(lens1)) / (2.0 * batch)
     out = {"tok_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3, "fill_s": fill_s, "mean_context": mean_ctx,
-           "graph_replays": c1["graph_replays"] - c0["graph_replays"]}
+           "graph_replays": c1["graph_replays"] - c0["graph_replays"], "ms_per_step_events": e0.elapsed_time(e1) / steps}
     for r in reqs:
         eng.abort(r)
     assert llm.cache.all_free()
     return out
+
+
+def bench_generate(llm, batch: int, prompt_len: int, new_tokens: int, seed: int) -> dict:
+    """The decode phase of the workload the shape is quoted with: ``batch`` requests, each a prompt of
+    ``prompt_len`` random tokens and ``new_tokens`` generated ones.  Prompts are prefilled under the
+    engine's token budget (requests admitted early decode meanwhile); the timed steps are those
+    from the moment every prompt is cached until the first request ends, so each of them decodes
+    one token for every one of the ``batch`` requests."""
+    import torch
+
+    from tensorline_amd import SamplingParams
+    cfg, eng = llm.model_config, llm.engine
+    reqs = [eng.add_request(p, SamplingParams(max_tokens=new_tokens, stop_token_ids={-1}))
+            for p in random_prompts(batch, prompt_len, cfg.vocab_size, seed)]
+    while any(r.num_computed < r.prompt_len for r in reqs):
+        eng.step()
+    sync()                                                  # every request has its first token; all decode from here
+    assert all(not r.done for r in reqs) and len(eng.scheduler.running) == batch
+    steps = new_tokens - max(r.num_generated for r in reqs)
+    lens0 = [len(r.tokens) for r in reqs]
+    g0 = eng.tokens_generated
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        eng.step()
+    e1.record()
+    sync()
+    dt = time.perf_counter() - t0
+    lens1 = [len(r.tokens) for r in reqs]
+    assert eng.tokens_generated - g0 == batch * steps and all(b - a == steps for a, b in zip(lens0, lens1))
+    eng.run_until_done()
+    assert all(r.done and r.num_generated == new_tokens for r in reqs) and llm.cache.all_free()
+    return {"tok_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3, "steps": steps,
+            "mean_context": (sum(lens0) + sum(lens1)) / (2.0 * batch), "ms_per_step_events": e0.elapsed_time(e1) / steps}
+
+
+def profile_decode_step(llm, batch: int, context: int, seed: int) -> dict:
+    """One decode step of ``batch`` sequences at about ``context`` tokens run eagerly, timed by class
+    of kernel with events around every launch (tensorline_amd/ops/profile.py)."""
+    from tensorline_amd import SamplingParams
+    from tensorline_amd.engine.runner import ModelRunner
+    from tensorline_amd.ops.profile import KernelTimer
+    cfg, eng = llm.model_config, llm.engine
+    prompt_len = context - 16 - (-(-batch * context // eng.scheduler.max_batched_tokens) if batch > 1 else 0)
+    reqs = [eng.add_request(p, SamplingParams(max_tokens=10 ** 9, stop_token_ids={-1}))
+            for p in random_prompts(batch, prompt_len, cfg.vocab_size, seed)]
+    while any(r.num_computed < r.prompt_len for r in reqs):
+        eng.step()
+    graph_runner, eager = eng.runner, ModelRunner(llm.model, llm.cache)
+    eager.fit_context = graph_runner.fit_context
+    eng.runner = eager
+    try:
+        for _ in range(3):
+            eng.step()
+        timer = KernelTimer()
+        with timer.measuring():
+            eng.step()
+    finally:
+        eng.runner = graph_runner
+    for r in reqs:
+        eng.abort(r)
+    return timer.summary()
 
 
 def bench_prefill(llm, tokens: int, reps: int, seed: int) -> dict:
@@ -236,6 +308,9 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--no-fp32", action="store_true", help="skip the 32-bit point")
+    ap.add_argument("--fp32-layers", type=int, default=4, help="layers of the model the 32-bit point runs")
+    ap.add_argument("--profile", action="store_true", help="add the time of one eager decode step by class of kernel")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's heuristic choice of kernels for prompt portions")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (default: the 7B shape)")
@@ -268,15 +343,46 @@ def main() -> int:
     elem = 2 if args.dtype in ("bfloat16", "bf16") else 4
     dtype_key = "bfloat16" if elem == 2 else "float32"
 
+    def with_roofline(run: dict, batch: int, model_cfg=cfg, elem_size=elem) -> dict:
+        """tok/s, ms per step (wall clock and events), mean context and the share of the HBM peak of a decode run."""
+        gbps = decode_bytes(model_cfg, batch, int(run["mean_context"]), elem_size) / (run["ms_per_step"] / 1e3) / 1e9
+        return {"tok_s": round(run["tok_s"], 1), "ms": round(run["ms_per_step"], 4), "ms_events": round(run["ms_per_step_events"], 4),
+                "ctx": round(run["mean_context"], 1), "GBps": round(gbps, 1), "hbm_frac": round(gbps / HBM_GBPS, 4)}
+
     main_run = bench_decode(llm, args.batch, args.context, args.steps, args.warmup, args.seed + 1)
     pre = bench_prefill(llm, args.prefill_tokens, 3, args.seed + 2)
     points = {}
     if not args.no_points:
         for b in (1, 64):
             k = max(8, args.steps // 2)
-            points[f"decode_b{b}"] = round(bench_decode(llm, b, args.context, k, 4, args.seed + 3 + b)["tok_s"], 1)
+            r = with_roofline(bench_decode(llm, b, args.context, k, 4, args.seed + 3 + b), b)
+            points[f"decode_b{b}"] = r["tok_s"]
+            points.update({f"decode_b{b}_{key}": r[key] for key in ("ms", "ctx", "hbm_frac")})
+        # the workload the shape is quoted with: 2,048-token prompts, 256 generated tokens each
+        for b in (1, 8, 64):
+            r = with_roofline(bench_generate(llm, b, 2048, 256, args.seed + 100 + b), b)
+            points[f"gen_b{b}"] = r["tok_s"]
+            points.update({f"gen_b{b}_{key}": r[key] for key in ("ms", "ms_events", "ctx", "hbm_frac")})
+    profile = profile_decode_step(llm, args.batch, args.context, args.seed + 7) if args.profile else None
 
     machine = measure_machine(torch.bfloat16 if elem == 2 else torch.float32)
+    fp32 = None
+    if elem == 2 and not args.no_points and not args.no_fp32:
+        # the true 32-bit path at the same layer sizes, fewer layers: what the equality checks cost
+        del llm
+        torch.cuda.empty_cache()
+        cfg32 = make_config(args.fp32_layers, args.shape)
+        llm32 = LLM(config=cfg32, seed=args.seed, dtype="float32", device="cuda:0", block_size=page,
+                    num_blocks=8 * (-(-max_len // page)) + 8, max_num_seqs=8, max_batched_tokens=2048,
+                    max_model_len=max_len, graphs=not args.no_graphs, graph_warmup_tokens=0, prefix_caching=False)
+        pre32 = bench_prefill(llm32, args.prefill_tokens, 2, args.seed + 2)
+        dec32 = with_roofline(bench_decode(llm32, 8, 2304, 8, 2, args.seed + 9), 8, cfg32, 4)
+        fp32 = {"layers": cfg32.num_hidden_layers, "layers_of_shape": full_layers,
+                "prefill_tok_s": round(pre32["tok_s"], 1), "prefill_ms": round(pre32["s"] * 1e3, 3),
+                "prefill_frac": round(prefill_flops(cfg32, args.prefill_tokens) / pre32["s"] / PEAK_FLOPS["float32"], 4),
+                "decode_b8_tok_s": dec32["tok_s"], "decode_b8_ms": dec32["ms"], "decode_b8_ctx": dec32["ctx"],
+                "decode_b8_hbm_frac": dec32["hbm_frac"]}
+        del llm32
     step_s = main_run["ms_per_step"] / 1e3
     achieved = decode_bytes(cfg, args.batch, int(main_run["mean_context"]), elem) / step_s / 1e9
     flops = prefill_flops(cfg, args.prefill_tokens)
@@ -288,6 +394,7 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(main_run["ms_per_step"], 4),
+        "ms_per_step_gpu_events": round(main_run["ms_per_step_events"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -311,6 +418,10 @@ def main() -> int:
         "points": points,
         "machine": machine,
     }
+    if fp32 is not None:
+        line["fp32"] = fp32
+    if profile is not None:
+        line["profile"] = profile
     print(json.dumps(line))
     torch.cuda.synchronize()
     return 0
