@@ -26,20 +26,30 @@ class ModelRunner:
         self.device = model.device
         self._host: torch.Tensor | None = None       # pinned staging for the step's metadata
         self._dev: torch.Tensor | None = None
+        self._copied: torch.cuda.Event | None = None   # recorded after the last copy out of the staging buffer
         self.steps = 0
         self.fit_context = 0          # the longest context this runner's engine allows, if it says so
 
     # ---- metadata ------------------------------------------------------------------------
     def _upload(self, data: np.ndarray) -> torch.Tensor:
         n = int(data.size)
+        pin = torch.device(self.device).type == "cuda"
         if self._dev is None or self._dev.numel() < n:
+            if self._copied is not None:
+                self._copied.synchronize()
             cap = max(4096, 1 << (max(n, 1) - 1).bit_length())
-            pin = torch.device(self.device).type == "cuda"
             self._host = torch.empty(cap, dtype=torch.int32, pin_memory=pin)
             self._dev = torch.empty(cap, dtype=torch.int32, device=self.device)
+        if self._copied is not None:
+            self._copied.synchronize()    # the last copy out of the staging buffer was only queued: wait before writing it again
         self._host[:n].numpy()[:] = data
-        # A blocking copy: the staging buffer is free for the next step when this returns.
-        self._dev[:n].copy_(self._host[:n], non_blocking=False)
+        if pin:
+            self._dev[:n].copy_(self._host[:n], non_blocking=True)
+            if self._copied is None:
+                self._copied = torch.cuda.Event()
+            self._copied.record()
+        else:
+            self._dev[:n].copy_(self._host[:n])
         return self._dev
 
     def pack(self, entries: Sequence[StepEntry], pad_seqs: int = 0, pad_nb: Sequence[int] | None = None) -> PackedBatch:

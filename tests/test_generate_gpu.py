@@ -356,9 +356,44 @@ def test_graph_replay_of_wide_buckets_matches_plain(case, rows, bucket, dtype):
             assert err < LIMIT[dtype], f"row {r} step {k}: relative error {err:.3e}"
             worst = max(worst, err)
     print(f"config {case.name} graph of {bucket} rows, {rows} live, {dtype}: worst relative error {worst:.3e}")
-    assert runner.graph_replays == steps - 1 and list(runner.graphs) == [bucket]
+    assert runner.graph_replays == steps - 1 and [b for b, c in runner.graphs] == [bucket]
     assert torch.all(cache.storage(0)["k"][bystander] == 7.0)
     assert torch.all(cache.storage(len(model.schedule) - 1)["v"][bystander] == -3.0)
+
+
+def test_decoding_across_a_context_bucket_switches_graphs_and_keeps_the_logits(folder_b):
+    """Graphs are captured per batch bucket and per context bucket (4,096 keys, then the engine's
+    limit): a request decoding from 4,090 to 4,110 tokens replays two graphs, and its logits are
+    those of the eager step to the bit and the plain implementation's within the bfloat16 limit."""
+    from tensorline_amd.cache.manager import CacheManager
+    from tensorline_amd.engine.batch import StepEntry
+    from tensorline_amd.engine.graphs import GraphRunner
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.runner import ModelRunner
+    d, w, cfg = folder_b
+    model, _ = load_model(d, "bfloat16", DEV)
+    limit_tokens, page = 4200, 8
+    toks = helpers.prompts_for("B", [4111], seed=12)[0]
+    want = plain.model_forward(w, cfg, toks)[4089:].numpy()
+    mk = lambda: CacheManager(model.cache_needs(), model.schedule, model.state_needs(), page_size=page,
+                              num_blocks=limit_tokens // page + 4, max_requests=2, dtype=model.dtype, device=DEV)
+    ce, cg = mk(), mk()
+    eager, graph = ModelRunner(model, ce), GraphRunner(model, cg, max_batch=2, max_blocks_per_seq=limit_tokens // page)
+    eager.fit_context = graph.fit_context
+    assert graph.context_buckets == [4096, limit_tokens]
+    for c, r in ((ce, eager), (cg, graph)):
+        c.add_request("a")
+        assert c.grow("a", len(toks))
+        for start in range(0, 4090, 1024):                      # the prompt in portions: eager either way
+            n = min(1024, 4090 - start)
+            r.step([StepEntry("a", toks[start:start + n], start, [])])
+    for pos in range(4090, len(toks)):
+        entry = [StepEntry("a", [toks[pos]], pos, [0])]
+        le, lg = eager.step(entry).clone(), graph.step(entry).clone()
+        torch.testing.assert_close(lg, le, atol=0, rtol=0)
+        err = float(np.abs(lg[0].cpu().numpy() - want[pos - 4089]).max()) / float(np.abs(want).max())
+        assert err < LIMIT["bfloat16"], (pos, err)
+    assert sorted(graph.graphs) == [(1, 4096), (1, limit_tokens)] and graph.graph_replays == len(toks) - 4090
 
 
 def test_parts_alone(folder_b):
