@@ -1,147 +1,390 @@
-// Causal attention of the step's tokens over the paged cache, for any head size, group size and
-// storage type.  One work-group per (token, key/value head); the query heads that share the
-// key/value head are handled together, up to AG_GC at a time.
+// Causal attention of the step's tokens over the paged cache, for any head size that is a multiple
+// of 16 up to 256, any group size, any page size and both storage types; all arithmetic in float.
+// Products run on the matrix cores' float instruction (v_mfma_f32_16x16x4_f32: float in, float
+// out, no reduced precision anywhere): this is the attention of the true 32-bit path, and of
+// bfloat16 shapes the bfloat16 matrix-core kernel does not take.
 //
 // A token at position p of sequence s attends to keys [lo, p] of that sequence, lo = 0 or
 // p - window + 1 for a windowed layer, found through the sequence's row of the page table.  The
 // keys of the step's own tokens are already in the cache when this runs.  k_cache is
-// [pages, page, nkv, d]; v_cache is [pages, nkv, d, page].  Scores, the running
-// maximum, the sum and the accumulator are float (reference: tensorline/paged_attn.py:25-58,
-// tensorline/paged.py:233-238).  Key tiles start at lo, so the result for a position does not
-// depend on how the sequence was cut into steps.
+// [pages, page, nkv, d]; v_cache is [pages, nkv, d, page] (reference: tensorline/paged_attn.py:25-58,
+// tensorline/paged.py:233-238).
+//
+// One work-group of four waves takes up to AG_ROWS = 64 rows: the (token, query head) pairs of a run
+// of consecutive tokens of one sequence's portion and the query heads of one key/value head, a
+// wave 16 rows.  Keys are walked in tiles of KT (64, or 32 for heads above 128) that start at
+// absolute multiples of KT.  A tile's keys and values are moved in 16-byte pieces, from the cache
+// into registers a tile ahead and from there as float into LDS: keys as [key][d], values as
+// [d][key], which is how the cache holds a page's values.  A wave computes S = Q K^T for its 16 rows
+// in blocks of 16 keys, the softmax of the tile per row (row maximum and sum by butterflies over
+// the 16 lanes that hold a row), rescales what it has summed so far (online softmax), passes P
+// through LDS into operand layout and adds P V.  Every sum runs in an order fixed by absolute key
+// positions and by the row alone, so the result for a position depends neither on how the
+// sequence was cut into steps nor on what else is in the batch.
+//
+// Operand layout of the 16x16x4 product D = A B + C: lane l gives A[l % 16][l / 16] and
+// B[l / 16][l % 16]; it holds D[4 (l / 16) + v][l % 16] in register v.  The four k of one product
+// need not be neighbours: here lane group g = l / 16 feeds k = 16 kk + 4 g + v to the v-th of four
+// products, for A and B alike, so that each lane's four operands are one 16-byte read.
 #include "common.h"
 
 #define AG_THREADS 256
-#define AG_TILE 256   // keys per tile, one per thread in the score phase
-#define AG_GC 8       // query heads per pass
+#define AG_ROWS 64
+#define AG_WROWS 16   // rows per wave
+
+#define AG_MAXC 8     // 16-byte pieces of a tile's keys (and of its values) a thread moves
 
 template <typename T>
+__device__ __forceinline__ float ag_load(const T* p) { return tl_to_float(*p); }
+
+// A 16-byte piece of the cache as floats: four of them, or eight bfloat16.
+template <typename T> struct AgPiece;
+template <> struct AgPiece<float> {
+    static constexpr int E = 4;
+    static __device__ __forceinline__ void unpack(const uint4& raw, float* f) {
+        f[0] = __uint_as_float(raw.x);
+        f[1] = __uint_as_float(raw.y);
+        f[2] = __uint_as_float(raw.z);
+        f[3] = __uint_as_float(raw.w);
+    }
+};
+template <> struct AgPiece<bf16_t> {
+    static constexpr int E = 8;
+    static __device__ __forceinline__ void unpack(const uint4& raw, float* f) {
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(w[i] << 16);
+            f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+};
+
+typedef float ag_f32x4 __attribute__((ext_vector_type(4)));
+
+// All lanes of a group of 16 get the same bits: every step adds a value to its mirror image.
+__device__ __forceinline__ float ag_row16_max(float v) {
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, TL_WAVE));
+    return v;
+}
+__device__ __forceinline__ float ag_row16_sum(float v) {
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) v += __shfl_xor(v, off, TL_WAVE);
+    return v;
+}
+
+// LDS: Ks [KT][d + 4] | Vt [d][KT + 4] | Ps [4 waves][16][KT + 4] | row_pos [64] | row_lo [64]
+template <typename T, int DB>    // DB: blocks of 16 head dimensions (d / 16), 1..16
 __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-    const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ seq_of_token,
-    const int32_t* __restrict__ pos, T* __restrict__ out, int out_stride, int nq, int nkv, int d, int dpad, int bs,
+    const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
+    T* __restrict__ out, int out_stride, int tiles_per_seq, int QT, int GC, int nq, int nkv, int bs, int KT,
     int window, float scale) {
+    constexpr int d = DB * 16;
     extern __shared__ float smem[];
-    float* q_s = smem;                         // [AG_GC][d]
-    float* s_s = q_s + AG_GC * d;              // [AG_GC][AG_TILE]
-    float* red = s_s + AG_GC * AG_TILE;        // [16]
-    float* acc_s = red + 16;                   // [AG_THREADS] for the final cross-subset sum
-    int* blk_s = (int*)(acc_s + AG_THREADS);   // [AG_TILE] cache row index of each key of the tile
+    constexpr int ks_ld = d + 4;
+    const int vt_ld = KT + 4, ps_ld = KT + 4;
+    float* Ks = smem;
+    float* Vt = Ks + KT * ks_ld;
+    float* Ps = Vt + d * vt_ld;
+    int* row_pos = reinterpret_cast<int*>(Ps + 4 * AG_WROWS * ps_ld);
+    int* row_lo = row_pos + AG_ROWS;
 
-    const int tid = threadIdx.x;
-    const int t = blockIdx.x, kvh = blockIdx.y;
-    const int s = seq_of_token[t];
-    const int p = pos[t];
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    const int hi = p + 1;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, lg = lane >> 4;             // position in the group of 16, and the group
+    const int s = blockIdx.x / tiles_per_seq, ti = blockIdx.x - s * tiles_per_seq;
+    const int kvh = blockIdx.y;
     const int G = nq / nkv;
+    const int g0 = blockIdx.z * GC;                       // first query head of this chunk within the group
+    const int gc = (G - g0 < GC) ? G - g0 : GC;
+    const int t_first = q_start[s] + ti * QT, t_end = q_start[s + 1];
+    if (t_first >= t_end) return;
+    const int nt = (t_end - t_first < QT) ? t_end - t_first : QT;
     const int32_t* table = tables + (size_t)s * NB;
 
-    // value phase mapping: thread = (dim c, key subset sub)
-    const int nsub = AG_THREADS / dpad;
-    const int c = tid % dpad, sub = tid / dpad;
+    // rows: r = i * GC + g for token i of the tile and head g of the chunk; others are padding
+    if (tid < AG_ROWS) {
+        const int i = tid / GC, g = tid - i * GC;
+        int p = -1, lo = 0;
+        if (i < nt && g < gc) {
+            p = pos[t_first + i];
+            lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+        }
+        row_pos[tid] = p;
+        row_lo[tid] = lo;
+    }
+    __syncthreads();
 
-    for (int g0 = 0; g0 < G; g0 += AG_GC) {
-        const int gc = (G - g0 < AG_GC) ? G - g0 : AG_GC;
-        for (int i = tid; i < gc * d; i += AG_THREADS) {
-            const int g = i / d, cc = i - g * d;
-            q_s[g * d + cc] = tl_to_float(q[(size_t)t * q_stride + (size_t)(kvh * G + g0 + g) * d + cc]) * scale;
+    // the keys any row of the tile sees, [k_lo, k_hi), and those the rows of this wave see
+    int k_lo = 0x7fffffff, k_hi = 0, w_lo = 0x7fffffff, w_hi = 0;
+    for (int r = 0; r < AG_ROWS; ++r) {
+        const int p = row_pos[r];
+        if (p < 0) continue;
+        const int lo = row_lo[r];
+        k_lo = (lo < k_lo) ? lo : k_lo;
+        k_hi = (p + 1 > k_hi) ? p + 1 : k_hi;
+        if (r / AG_WROWS == wave) {
+            w_lo = (lo < w_lo) ? lo : w_lo;
+            w_hi = (p + 1 > w_hi) ? p + 1 : w_hi;
         }
-        float m[AG_GC], l[AG_GC], acc[AG_GC];
-#pragma unroll
-        for (int g = 0; g < AG_GC; ++g) {
-            m[g] = -INFINITY;
-            l[g] = 0.f;
-            acc[g] = 0.f;
-        }
-        __syncthreads();
+    }
 
-        for (int k0 = lo; k0 < hi; k0 += AG_TILE) {
-            const int key = k0 + tid;
-            const bool valid = key < hi;
-            float sc[AG_GC];
+    // A operand of S = Q K^T: this lane's row is li of the wave's 16; scaled queries, kept in registers
+    ag_f32x4 qa[DB];
+    {
+        const int row = wave * AG_WROWS + li;
+        const int i = row / GC, g = row - i * GC;
+        const bool real = row_pos[row] >= 0;
+        const T* qrow = q + (size_t)(t_first + (real ? i : 0)) * q_stride + (size_t)(kvh * G + g0 + (real ? g : 0)) * d;
 #pragma unroll
-            for (int g = 0; g < AG_GC; ++g) sc[g] = 0.f;
-            if (valid) {
-                const int blk = table[key / bs];
-                const int row = blk * bs + key % bs;
-                blk_s[tid] = row;
-                const T* kr = k_cache + ((size_t)row * nkv + kvh) * d;
-                for (int cc = 0; cc < d; ++cc) {
-                    const float kv = tl_to_float(kr[cc]);
+        for (int kk = 0; kk < DB; ++kk) {
 #pragma unroll
-                    for (int g = 0; g < AG_GC; ++g)
-                        if (g < gc) sc[g] = fmaf(q_s[g * d + cc], kv, sc[g]);
-                }
-            } else {
-                blk_s[tid] = 0;
-            }
-#pragma unroll
-            for (int g = 0; g < AG_GC; ++g) {
-                if (g >= gc) break;
-                const float sv = valid ? sc[g] : -INFINITY;
-                const float mx = tl_block_max(sv, red);
-                const float m_new = fmaxf(m[g], mx);
-                const float alpha = expf(m[g] - m_new);   // exp(-inf) = 0 on the first tile
-                const float pe = valid ? expf(sv - m_new) : 0.f;
-                s_s[g * AG_TILE + tid] = pe;
-                const float psum = tl_block_sum(pe, red);
-                l[g] = l[g] * alpha + psum;
-                acc[g] *= alpha;
-                m[g] = m_new;
-            }
-            __syncthreads();
-            const int nkeys = (hi - k0 < AG_TILE) ? hi - k0 : AG_TILE;
-            if (c < d) {
-                for (int j = sub; j < nkeys; j += nsub) {
-                    const int vrow = blk_s[j];
-                    const float vv = tl_to_float(v_cache[(((size_t)(vrow / bs) * nkv + kvh) * d + c) * bs + vrow % bs]);
-#pragma unroll
-                    for (int g = 0; g < AG_GC; ++g)
-                        if (g < gc) acc[g] = fmaf(s_s[g * AG_TILE + j], vv, acc[g]);
-                }
-            }
-            __syncthreads();
+            for (int v = 0; v < 4; ++v) qa[kk][v] = real ? ag_load(qrow + 16 * kk + 4 * lg + v) * scale : 0.f;
         }
-        // sum the key subsets and write
-        for (int g = 0; g < gc; ++g) {
-            acc_s[tid] = acc[g];
-            __syncthreads();
-            if (sub == 0 && c < d) {
+    }
+    // the rows this lane holds of S and of the output: 4 lg + v
+    int my_pos[4], my_lo[4];
+    float m[4], l[4];
+    ag_f32x4 acc[DB];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        my_pos[v] = row_pos[wave * AG_WROWS + 4 * lg + v];
+        my_lo[v] = row_lo[wave * AG_WROWS + 4 * lg + v];
+        m[v] = -INFINITY;
+        l[v] = 0.f;
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) acc[db] = (ag_f32x4){0.f, 0.f, 0.f, 0.f};
+    float* Pw = Ps + wave * AG_WROWS * ps_ld;
+
+    // A tile's keys and values travel in 16-byte pieces: from the cache into registers (issued a tile
+    // ahead, so the loads are in flight while the tile before is computed), from there as float into LDS.
+    // Keys: a piece is E consecutive head dimensions of one key.  Values: E consecutive keys of one
+    // head dimension (one page holds them contiguously; needs a page size that is a multiple of E,
+    // otherwise values are fetched one by one).
+    constexpr int E = AgPiece<T>::E;
+    constexpr int cpr = d / E;                             // pieces per key
+    const int vpc = KT / E;                                // pieces per head dimension
+    const int pieces = KT * cpr;                           // == d * vpc, at most AG_MAXC * AG_THREADS
+    const bool v_pieces = (bs % E) == 0;
+    uint4 kreg[AG_MAXC], vreg[AG_MAXC];
+
+    // No branch in here: every piece is loaded from a valid address (indices clamped into the range
+    // the tile's rows see; what lies outside is zeroed on the way into LDS), so all page lookups are
+    // issued together and all cache loads after one wait.
+    auto fetch = [&](int k0) {
+        int krow[AG_MAXC], vpage[AG_MAXC];
+#pragma unroll
+        for (int it = 0; it < AG_MAXC; ++it) {
+            int qi = tid + it * AG_THREADS;
+            qi = (qi < pieces) ? qi : pieces - 1;
+            int key = k0 + qi / cpr;
+            key = (key < k_hi) ? key : k_hi - 1;
+            krow[it] = table[key / bs] * bs + key % bs;
+            const int c = qi / vpc;
+            int vkey = k0 + (qi - c * vpc) * E;
+            vkey = (vkey < k_hi) ? vkey : ((k_hi - 1) / E) * E;
+            vpage[it] = table[vkey / bs];
+        }
+#pragma unroll
+        for (int it = 0; it < AG_MAXC; ++it) {
+            int qi = tid + it * AG_THREADS;
+            qi = (qi < pieces) ? qi : pieces - 1;
+            const int j = qi / cpr, cc = qi - j * cpr;
+            kreg[it] = *reinterpret_cast<const uint4*>(k_cache + ((size_t)krow[it] * nkv + kvh) * d + cc * E);
+            if (v_pieces) {
+                const int c = qi / vpc;
+                int vkey = k0 + (qi - c * vpc) * E;
+                vkey = (vkey < k_hi) ? vkey : ((k_hi - 1) / E) * E;
+                vreg[it] = *reinterpret_cast<const uint4*>(v_cache + (((size_t)vpage[it] * nkv + kvh) * d + c) * bs + vkey % bs);
+            }
+        }
+    };
+    auto to_lds = [&](int k0) {
+#pragma unroll
+        for (int it = 0; it < AG_MAXC; ++it) {
+            const int qi = tid + it * AG_THREADS;
+            if (qi >= pieces) continue;
+            float f[E];
+            const int j = qi / cpr, cc = qi - j * cpr;
+            AgPiece<T>::unpack(kreg[it], f);
+            const bool key_seen = k0 + j < k_hi;
+#pragma unroll
+            for (int e = 0; e < E; e += 4)
+                *reinterpret_cast<float4*>(Ks + j * ks_ld + cc * E + e) =
+                    key_seen ? make_float4(f[e], f[e + 1], f[e + 2], f[e + 3]) : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (v_pieces) {
+                const int c = qi / vpc, j0 = (qi - c * vpc) * E;
+                AgPiece<T>::unpack(vreg[it], f);
+#pragma unroll
+                for (int e = 0; e < E; ++e) f[e] = (k0 + j0 + e < k_hi) ? f[e] : 0.f;
+#pragma unroll
+                for (int e = 0; e < E; e += 4)
+                    *reinterpret_cast<float4*>(Vt + c * vt_ld + j0 + e) = make_float4(f[e], f[e + 1], f[e + 2], f[e + 3]);
+            }
+        }
+        if (!v_pieces) {
+            for (int idx = tid; idx < KT * d; idx += AG_THREADS) {
+                const int c = idx / KT, j = idx - c * KT;
+                const int key = k0 + j;
                 float v = 0.f;
-                for (int u = 0; u < nsub; ++u) v += acc_s[u * dpad + c];
-                out[(size_t)t * out_stride + (size_t)(kvh * G + g0 + g) * d + c] = tl_from_float<T>(v / l[g]);
+                if (key < k_hi) {
+                    const int page = table[key / bs];
+                    v = ag_load(v_cache + (((size_t)page * nkv + kvh) * d + c) * bs + key % bs);
+                }
+                Vt[c * vt_ld + j] = v;
             }
-            __syncthreads();
         }
+    };
+
+    const int k_first = (k_lo / KT) * KT;
+    const int key_blocks = KT / 16;
+    fetch(k_first);
+    for (int k0 = k_first; k0 < k_hi; k0 += KT) {
+        to_lds(k0);
+        __syncthreads();
+        if (k0 + KT < k_hi) fetch(k0 + KT);
+
+        if (k0 < w_hi && k0 + KT > w_lo) {                 // a tile none of the wave's rows sees is skipped
+            // ---- S = Q K^T: per block of 16 keys, 4 DB products; lane holds rows 4 lg + v, key li ----
+            ag_f32x4 sblk[4];
+#pragma unroll
+            for (int jb = 0; jb < 4; ++jb) {
+                sblk[jb] = (ag_f32x4){0.f, 0.f, 0.f, 0.f};
+                if (jb < key_blocks) {
+                    const float* kr = Ks + (jb * 16 + li) * ks_ld + 4 * lg;
+#pragma unroll
+                    for (int kk = 0; kk < DB; ++kk) {
+                        const float4 kb = *reinterpret_cast<const float4*>(kr + 16 * kk);
+                        sblk[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk][0], kb.x, sblk[jb], 0, 0, 0);
+                        sblk[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk][1], kb.y, sblk[jb], 0, 0, 0);
+                        sblk[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk][2], kb.z, sblk[jb], 0, 0, 0);
+                        sblk[jb] = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[kk][3], kb.w, sblk[jb], 0, 0, 0);
+                    }
+                }
+            }
+            // ---- softmax over the tile, per row; rescale what was summed so far ----------------------
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                float sv[4], mx = -INFINITY;
+#pragma unroll
+                for (int jb = 0; jb < 4; ++jb) {
+                    const int key = k0 + jb * 16 + li;
+                    const bool seen = jb < key_blocks && my_pos[v] >= 0 && key <= my_pos[v] && key >= my_lo[v];
+                    sv[jb] = seen ? sblk[jb][v] : -INFINITY;
+                    mx = fmaxf(mx, sv[jb]);
+                }
+                const float m_new = fmaxf(m[v], ag_row16_max(mx));
+                float alpha = 1.f, psum = 0.f;
+                if (m_new > -INFINITY) {                   // else: the row sees no key yet
+                    alpha = expf(m[v] - m_new);            // exp(-inf) = 0 for the first tile the row sees
+#pragma unroll
+                    for (int jb = 0; jb < 4; ++jb) {
+                        sv[jb] = (sv[jb] > -INFINITY) ? expf(sv[jb] - m_new) : 0.f;
+                        psum += sv[jb];
+                    }
+                } else {
+#pragma unroll
+                    for (int jb = 0; jb < 4; ++jb) sv[jb] = 0.f;
+                }
+                l[v] = l[v] * alpha + ag_row16_sum(psum);
+                m[v] = m_new;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) acc[db][v] *= alpha;
+#pragma unroll
+                for (int jb = 0; jb < 4; ++jb)
+                    if (jb < key_blocks) Pw[(4 * lg + v) * ps_ld + jb * 16 + li] = sv[jb];
+            }
+            // Pw is written and read by this wave only; LDS operations of a wave complete in order
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // ---- O += P V: A = P (row li, keys 16 kk + 4 lg + v), B = values (keys likewise, dimension li) ----
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                if (kk < key_blocks) {
+                    const float4 pa = *reinterpret_cast<const float4*>(Pw + li * ps_ld + 16 * kk + 4 * lg);
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) {
+                        const float4 vb = *reinterpret_cast<const float4*>(Vt + (db * 16 + li) * vt_ld + 16 * kk + 4 * lg);
+                        acc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa.x, vb.x, acc[db], 0, 0, 0);
+                        acc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa.y, vb.y, acc[db], 0, 0, 0);
+                        acc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa.z, vb.z, acc[db], 0, 0, 0);
+                        acc[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa.w, vb.w, acc[db], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        __syncthreads();                                   // the tile is used up: the next one may be loaded
+    }
+
+    // this lane holds output rows 4 lg + v at head dimensions 16 db + li
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        if (my_pos[v] < 0) continue;
+        const int row = wave * AG_WROWS + 4 * lg + v;
+        const int i = row / GC, g = row - i * GC;
+        const float inv = (l[v] > 0.f) ? 1.f / l[v] : 0.f;
+        T* orow = out + (size_t)(t_first + i) * out_stride + (size_t)(kvh * G + g0 + g) * d;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) orow[db * 16 + li] = tl_from_float<T>(acc[db][v] * inv);
     }
 }
 
+static size_t ag_lds_bytes(int d, int KT) {
+    return sizeof(float) * ((size_t)KT * (d + 4) + (size_t)d * (KT + 4) + 4 * AG_WROWS * (KT + 4)) + sizeof(int) * (2 * AG_ROWS);
+}
+
+// q_start: int32 [S + 1], the first row of each sequence in the flat batch (rows of a sequence are
+// consecutive); max_query_len: the most tokens one sequence brings to this step.
 extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_cache, const void* v_cache,
-                                    const int32_t* tables, int NB, const int32_t* seq_of_token, const int32_t* pos,
-                                    void* out, int out_stride, int dtype, int T, int nq, int nkv, int d, int bs,
-                                    int window, float scale, hipStream_t stream) {
-    TL_CHECK_ARG(T >= 0 && nq > 0 && nkv > 0 && d > 0 && bs > 0 && NB > 0,
-                 "tl_attention_generic: bad sizes T=%d nq=%d nkv=%d d=%d page=%d NB=%d", T, nq, nkv, d, bs, NB);
+                                    const int32_t* tables, int NB, const int32_t* q_start, const int32_t* pos,
+                                    void* out, int out_stride, int dtype, int T, int S, int max_query_len, int nq, int nkv,
+                                    int d, int bs, int window, float scale, hipStream_t stream) {
+    TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && d > 0 && bs > 0 && NB > 0,
+                 "tl_attention_generic: bad sizes T=%d S=%d nq=%d nkv=%d d=%d page=%d NB=%d", T, S, nq, nkv, d, bs, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_generic: %d query heads are not a multiple of %d key/value heads", nq, nkv);
-    TL_CHECK_ARG(d <= 256, "tl_attention_generic: head size %d is above the supported 256", d);
+    TL_CHECK_ARG(d <= 256 && d % 16 == 0, "tl_attention_generic: head size %d must be a multiple of 16 and at most 256", d);
     TL_CHECK_ARG(nkv <= 65535, "tl_attention_generic: too many key/value heads %d", nkv);
     TL_CHECK_ARG(q_stride >= nq * d && out_stride >= nq * d, "tl_attention_generic: row strides too small");
-    if (T == 0) return 0;
-    int dpad = 1;
-    while (dpad < d) dpad <<= 1;
-    const size_t smem = sizeof(float) * ((size_t)AG_GC * d + (size_t)AG_GC * AG_TILE + 16 + AG_THREADS) + sizeof(int) * AG_TILE;
-    dim3 grid(T, nkv), block(AG_THREADS);
-    if (dtype == TL_F32)
-        hipLaunchKernelGGL(attn_generic_kernel<float>, grid, block, smem, stream, (const float*)q, q_stride,
-                           (const float*)k_cache, (const float*)v_cache, tables, NB, seq_of_token, pos, (float*)out,
-                           out_stride, nq, nkv, d, dpad, bs, window, scale);
-    else if (dtype == TL_BF16)
-        hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, block, smem, stream, (const bf16_t*)q, q_stride,
-                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, tables, NB, seq_of_token, pos, (bf16_t*)out,
-                           out_stride, nq, nkv, d, dpad, bs, window, scale);
-    else
+    TL_CHECK_ARG(max_query_len >= 1 || T == 0, "tl_attention_generic: max_query_len %d", max_query_len);
+    if (T == 0 || S == 0) return 0;
+    const int G = nq / nkv;
+    const int GC = (G < AG_ROWS) ? G : AG_ROWS;           // query heads per work-group
+    const int QT = AG_ROWS / GC;                          // tokens per work-group
+    const int chunks = tl_ceil_div(G, GC);
+    TL_CHECK_ARG(chunks <= 65535, "tl_attention_generic: group of %d query heads is too large", G);
+    const int tiles_per_seq = tl_ceil_div(max_query_len, QT);
+    const long long groups = (long long)S * tiles_per_seq;
+    TL_CHECK_ARG(groups <= 0x7fffffffLL, "tl_attention_generic: too many work-groups");
+    const int KT = (d <= 128) ? 64 : 32;
+    const size_t smem = ag_lds_bytes(d, KT);
+    TL_CHECK_ARG(smem <= 160 * 1024, "tl_attention_generic: head size %d needs %zu bytes of LDS", d, smem);
+    TL_CHECK_ARG(KT * d / 4 <= AG_MAXC * AG_THREADS, "tl_attention_generic: a tile of head size %d has too many pieces", d);
+    dim3 grid((unsigned)groups, nkv, chunks), block(AG_THREADS);
+#define AG_LAUNCH(TT, DB)                                                                                             \
+    hipLaunchKernelGGL((attn_generic_kernel<TT, DB>), grid, block, smem, stream, (const TT*)q, q_stride,              \
+                       (const TT*)k_cache, (const TT*)v_cache, tables, NB, q_start, pos, (TT*)out, out_stride,          \
+                       tiles_per_seq, QT, GC, nq, nkv, bs, KT, window, scale)
+#define AG_CASE(TT, DB) \
+    case DB: AG_LAUNCH(TT, DB); break;
+#define AG_DISPATCH(TT)                                                                              \
+    switch (d / 16) {                                                                                \
+        AG_CASE(TT, 1) AG_CASE(TT, 2) AG_CASE(TT, 3) AG_CASE(TT, 4) AG_CASE(TT, 5) AG_CASE(TT, 6)      \
+        AG_CASE(TT, 7) AG_CASE(TT, 8) AG_CASE(TT, 9) AG_CASE(TT, 10) AG_CASE(TT, 11) AG_CASE(TT, 12)  \
+        AG_CASE(TT, 13) AG_CASE(TT, 14) AG_CASE(TT, 15) AG_CASE(TT, 16)                               \
+    }
+    if (dtype == TL_F32) {
+        AG_DISPATCH(float)
+    } else if (dtype == TL_BF16) {
+        AG_DISPATCH(bf16_t)
+    } else {
         return tl_fail("tl_attention_generic: unknown dtype %d", dtype);
+    }
+#undef AG_DISPATCH
+#undef AG_CASE
+#undef AG_LAUNCH
     TL_CHECK_LAUNCH("tl_attention_generic");
     return 0;
 }

@@ -686,8 +686,20 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
               num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,
               0 if path == "mfma-direct" else 1, total128, _ptr(None), 0, skip_single, _stream())
         return out
+    # The any-shape kernel tiles each sequence's tokens: it needs the first row of every sequence and the
+    # most tokens one of them brings.  The engine has both; a bare call derives them from seq_of_token.
+    S = tables.shape[0]
+    if q_start is not None and plan is not None:
+        _i32(q_start, "q_start", S + 1)
+        max_query_len = int(plan.max_query_len)
+    else:
+        counts = torch.bincount(seq_of_token.long(), minlength=S)[:S]
+        q_start = torch.zeros(S + 1, dtype=torch.int32, device=q.device)
+        q_start[1:] = torch.cumsum(counts, 0)
+        max_query_len = int(counts.max().item()) if T else 1
+    _check(head_dim % 16 == 0 and head_dim <= 256, f"paged_attention: head size {head_dim} must be a multiple of 16, at most 256")
     _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
-          _ptr(seq_of_token), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, num_heads,
+          _ptr(q_start), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, S, max(max_query_len, 1), num_heads,
           num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), _stream())
     return out
 
