@@ -1,67 +1,184 @@
-// C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]):  the plain tiled matrix product.
+// C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]):  the any-shape matrix product.
 //
-// This is the true 32-bit path (float inputs, float FMA, float accumulation in a fixed order over
-// k, no reduced-precision matrix mode) and the any-shape fallback for bfloat16 inputs.  The order
-// of accumulation of one output element does not depend on M, so cutting a batch differently does
-// not change a result.
+// This is the product of the true 32-bit path (float inputs, float products and sums on the matrix
+// cores' float instruction v_mfma_f32_16x16x4_f32, no reduced precision anywhere) and the any-shape
+// fallback for bfloat16 inputs (converted to float on the way into LDS, which is exact).  Any M, N
+// and K, any row strides.
+//
+// One output element is summed over k in one fixed order: steps of 16 from k = 0 upwards, four
+// products per step, the lanes' k within a step fixed by the operand layout.  The order does not
+// depend on M or on which tile shape the launch picked, so cutting a batch differently does not
+// change a bit of a result, and neither does the number of rows that come along.
+//
+// Tiles: four waves compute BM x BN outputs, a wave MB x NB blocks of 16 x 16; 128 x 128 for many
+// rows, 64 x 128 and 32 x 64 for few (more work-groups stream the weights then).  A k-step's rows
+// of A and W go from memory into registers while the step before is computed, then as float into
+// LDS [row][16 + 4] (the padding keeps the 16-byte operand reads off each other's banks).
+//
+// Operand layout of the 16x16x4 product D = A B + C: lane l gives A[l % 16][l / 16] and
+// B[l / 16][l % 16]; it holds D[4 (l / 16) + v][l % 16] in register v.  Lane group g = l / 16 feeds
+// k = 4 g + v of the step to the v-th of its four products, for A and B alike, so a lane's four
+// operands are one 16-byte read.
 #include "common.h"
 
-#define GT_BM 64
-#define GT_BN 64
-#define GT_BK 16
+#define GG_THREADS 256
+#define GG_KS 16              // k per step
+#define GG_LD (GG_KS + 4)     // LDS row stride in floats
+
+typedef float gg_f32x4 __attribute__((ext_vector_type(4)));
+
+// Four consecutive k of one row as floats; zero where the row or k is outside the matrix.
+template <typename T>
+__device__ __forceinline__ float4 gg_load4(const T* __restrict__ base, bool row_ok, int k, int K, bool vec_ok);
+
+template <>
+__device__ __forceinline__ float4 gg_load4<float>(const float* __restrict__ base, bool row_ok, int k, int K, bool vec_ok) {
+    if (!row_ok || k >= K) return make_float4(0.f, 0.f, 0.f, 0.f);
+    if (vec_ok && k + 3 < K) return *reinterpret_cast<const float4*>(base + k);
+    float4 r;
+    r.x = base[k];
+    r.y = (k + 1 < K) ? base[k + 1] : 0.f;
+    r.z = (k + 2 < K) ? base[k + 2] : 0.f;
+    r.w = (k + 3 < K) ? base[k + 3] : 0.f;
+    return r;
+}
+
+template <>
+__device__ __forceinline__ float4 gg_load4<bf16_t>(const bf16_t* __restrict__ base, bool row_ok, int k, int K, bool vec_ok) {
+    if (!row_ok || k >= K) return make_float4(0.f, 0.f, 0.f, 0.f);
+    if (vec_ok && k + 3 < K) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(base + k);
+        return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                           __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u));
+    }
+    float4 r;
+    r.x = tl_to_float(base[k]);
+    r.y = (k + 1 < K) ? tl_to_float(base[k + 1]) : 0.f;
+    r.z = (k + 2 < K) ? tl_to_float(base[k + 2]) : 0.f;
+    r.w = (k + 3 < K) ? tl_to_float(base[k + 3]) : 0.f;
+    return r;
+}
+
+// WM x WN waves (WM * WN == 4), each MB x NB blocks of 16 x 16.
+template <typename TA, typename TW, typename TO, int WM, int WN, int MB, int NB>
+__global__ __launch_bounds__(GG_THREADS) void gemm_generic_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
+                                                                 const float* __restrict__ bias, TO* __restrict__ C,
+                                                                 int M, int N, int K, int lda, int ldc, int a_vec,
+                                                                 int w_vec) {
+    constexpr int BM = WM * MB * 16, BN = WN * NB * 16;
+    constexpr int A_PIECES = BM * 4, W_PIECES = BN * 4;                 // 16-byte (four k) pieces per step
+    constexpr int A_PER = (A_PIECES + GG_THREADS - 1) / GG_THREADS, W_PER = (W_PIECES + GG_THREADS - 1) / GG_THREADS;
+    __shared__ float As[2][BM * GG_LD];
+    __shared__ float Ws[2][BN * GG_LD];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, lg = lane >> 4;
+    const int wm = wave / WN, wn = wave - wm * WN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+    gg_f32x4 acc[MB][NB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) acc[i][j] = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
+
+    float4 areg[A_PER], wreg[W_PER];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int it = 0; it < A_PER; ++it) {
+            const int p = tid + it * GG_THREADS;
+            const int r = p >> 2, c4 = p & 3;
+            areg[it] = gg_load4<TA>(A + (size_t)(m0 + r) * lda, p < A_PIECES && m0 + r < M, k0 + 4 * c4, K, a_vec != 0);
+        }
+#pragma unroll
+        for (int it = 0; it < W_PER; ++it) {
+            const int p = tid + it * GG_THREADS;
+            const int r = p >> 2, c4 = p & 3;
+            wreg[it] = gg_load4<TW>(W + (size_t)(n0 + r) * K, p < W_PIECES && n0 + r < N, k0 + 4 * c4, K, w_vec != 0);
+        }
+    };
+    auto to_lds = [&](int buf) {
+#pragma unroll
+        for (int it = 0; it < A_PER; ++it) {
+            const int p = tid + it * GG_THREADS;
+            if (p < A_PIECES) *reinterpret_cast<float4*>(&As[buf][(p >> 2) * GG_LD + 4 * (p & 3)]) = areg[it];
+        }
+#pragma unroll
+        for (int it = 0; it < W_PER; ++it) {
+            const int p = tid + it * GG_THREADS;
+            if (p < W_PIECES) *reinterpret_cast<float4*>(&Ws[buf][(p >> 2) * GG_LD + 4 * (p & 3)]) = wreg[it];
+        }
+    };
+
+    fetch(0);
+    to_lds(0);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += GG_KS) {
+        const bool more = k0 + GG_KS < K;
+        if (more) fetch(k0 + GG_KS);
+        float4 af[MB], wf[NB];
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+            af[i] = *reinterpret_cast<const float4*>(&As[buf][((wm * MB + i) * 16 + li) * GG_LD + 4 * lg]);
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+            wf[j] = *reinterpret_cast<const float4*>(&Ws[buf][((wn * NB + j) * 16 + li) * GG_LD + 4 * lg]);
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i].x, wf[j].x, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i].y, wf[j].y, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i].z, wf[j].z, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i].w, wf[j].w, acc[i][j], 0, 0, 0);
+            }
+        if (more) {
+            to_lds(buf ^ 1);          // the other buffer: nobody reads it during this step
+            __syncthreads();
+            buf ^= 1;
+        }
+    }
+
+    // this lane holds rows 4 lg + v and column li of each block
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int n = n0 + (wn * NB + j) * 16 + li;
+        if (n >= N) continue;
+        const float b = bias ? bias[n] : 0.f;
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int m = m0 + (wm * MB + i) * 16 + 4 * lg + v;
+                if (m < M) C[(size_t)m * ldc + n] = tl_from_float<TO>(acc[i][j][v] + b);
+            }
+    }
+}
 
 template <typename TA, typename TW, typename TO>
-__global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
-                                                          const float* __restrict__ bias, TO* __restrict__ C, int M,
-                                                          int N, int K, int lda, int ldc) {
-    __shared__ float As[GT_BK][GT_BM + 4];
-    __shared__ float Ws[GT_BK][GT_BN + 4];
-    const int tid = threadIdx.x;
-    const int m0 = blockIdx.y * GT_BM, n0 = blockIdx.x * GT_BN;
-    const int tx = tid & 15, ty = tid >> 4;  // 16 x 16 threads, 4 x 4 outputs each
-    const int lr = tid >> 2, lk = (tid & 3) * 4;  // loader: row lr of the tile, k offset lk..lk+3
-
-    float acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
-
-    for (int k0 = 0; k0 < K; k0 += GT_BK) {
-        const int am = m0 + lr, wn = n0 + lr;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int k = k0 + lk + j;
-            As[lk + j][lr] = (am < M && k < K) ? tl_to_float(A[(size_t)am * lda + k]) : 0.f;
-            Ws[lk + j][lr] = (wn < N && k < K) ? tl_to_float(W[(size_t)wn * K + k]) : 0.f;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < GT_BK; ++k) {
-            float a[4], w[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) w[j] = Ws[k][tx * 4 + j];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
-        }
-        __syncthreads();
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = m0 + ty * 4 + i;
-        if (m >= M) continue;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + tx * 4 + j;
-            if (n >= N) continue;
-            const float v = acc[i][j] + (bias ? bias[n] : 0.f);
-            C[(size_t)m * ldc + n] = tl_from_float<TO>(v);
-        }
-    }
+static int gg_launch(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, int lda, int ldc,
+                     hipStream_t stream) {
+    // whole 16-byte (8-byte for bfloat16) pieces can be read where rows start aligned
+    const int a_vec = ((uintptr_t)A % (4 * sizeof(TA)) == 0 && lda % 4 == 0) ? 1 : 0;
+    const int w_vec = ((uintptr_t)W % (4 * sizeof(TW)) == 0 && K % 4 == 0) ? 1 : 0;
+#define GG_GO(WM, WN, MB, NB)                                                                                    \
+    do {                                                                                                         \
+        constexpr int BM = WM * MB * 16, BN = WN * NB * 16;                                                      \
+        const long long gy = tl_ceil_div(M, BM);                                                                 \
+        if (gy > 65535) return tl_fail("tl_gemm_generic: %d rows are too many for one launch", M);               \
+        dim3 grid(tl_ceil_div(N, BN), (unsigned)gy), block(GG_THREADS);                                          \
+        hipLaunchKernelGGL((gemm_generic_kernel<TA, TW, TO, WM, WN, MB, NB>), grid, block, 0, stream,            \
+                           (const TA*)A, (const TW*)W, bias, (TO*)C, M, N, K, lda, ldc, a_vec, w_vec);           \
+    } while (0)
+    if (M <= 32)
+        GG_GO(1, 4, 2, 1);        // 32 x 64
+    else if (M <= 64)
+        GG_GO(1, 4, 4, 2);        // 64 x 128
+    else
+        GG_GO(2, 2, 4, 4);        // 128 x 128
+#undef GG_GO
+    return 0;
 }
 
 // A: [M, K] with row stride lda; W: [N, K] contiguous; C: [M, N] with row stride ldc.
@@ -70,23 +187,18 @@ extern "C" int tl_gemm_generic(const void* A, int a_dtype, const void* W, int w_
     TL_CHECK_ARG(M >= 0 && N > 0 && K > 0, "tl_gemm_generic: bad sizes M=%d N=%d K=%d", M, N, K);
     TL_CHECK_ARG(lda >= K && ldc >= N, "tl_gemm_generic: row strides lda=%d ldc=%d too small for K=%d N=%d", lda, ldc, K, N);
     if (M == 0) return 0;
-    for (int m0 = 0; m0 < M; m0 += 65535 * GT_BM) {  // grid.y limit
-        const int mm = (M - m0 < 65535 * GT_BM) ? M - m0 : 65535 * GT_BM;
-        dim3 grid(tl_ceil_div(N, GT_BN), tl_ceil_div(mm, GT_BM)), block(256);
-#define TL_GEMM_CASE(AD, AT, WD, WT, CD, CT)                                                                     \
-    if (a_dtype == AD && w_dtype == WD && c_dtype == CD) {                                                       \
-        hipLaunchKernelGGL((gemm_generic_kernel<AT, WT, CT>), grid, block, 0, stream,                            \
-                           (const AT*)A + (size_t)m0 * lda, (const WT*)W, bias, (CT*)C + (size_t)m0 * ldc, mm, N, K, \
-                           lda, ldc);                                                                            \
-        continue;                                                                                                \
-    }
-        TL_GEMM_CASE(TL_F32, float, TL_F32, float, TL_F32, float)
-        TL_GEMM_CASE(TL_BF16, bf16_t, TL_BF16, bf16_t, TL_BF16, bf16_t)
-        TL_GEMM_CASE(TL_BF16, bf16_t, TL_BF16, bf16_t, TL_F32, float)
-        TL_GEMM_CASE(TL_F32, float, TL_BF16, bf16_t, TL_F32, float)
-#undef TL_GEMM_CASE
+    int rc;
+    if (a_dtype == TL_F32 && w_dtype == TL_F32 && c_dtype == TL_F32)
+        rc = gg_launch<float, float, float>(A, W, bias, C, M, N, K, lda, ldc, stream);
+    else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_BF16)
+        rc = gg_launch<bf16_t, bf16_t, bf16_t>(A, W, bias, C, M, N, K, lda, ldc, stream);
+    else if (a_dtype == TL_BF16 && w_dtype == TL_BF16 && c_dtype == TL_F32)
+        rc = gg_launch<bf16_t, bf16_t, float>(A, W, bias, C, M, N, K, lda, ldc, stream);
+    else if (a_dtype == TL_F32 && w_dtype == TL_BF16 && c_dtype == TL_F32)
+        rc = gg_launch<float, bf16_t, float>(A, W, bias, C, M, N, K, lda, ldc, stream);
+    else
         return tl_fail("tl_gemm_generic: unsupported dtypes a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
-    }
+    if (rc) return rc;
     TL_CHECK_LAUNCH("tl_gemm_generic");
     return 0;
 }
