@@ -108,6 +108,7 @@ def bench_decode(llm, batch: int, context: int, steps: int, warmup: int, seed: i
     fill_s = time.perf_counter() - t0
     for _ in range(warmup):
         eng.step()
+    eng.drain()                                                      # nothing in flight when the clock starts
     sync()
     assert all(not r.done for r in reqs) and len(eng.scheduler.running) == batch and not eng.scheduler.waiting
     import torch
@@ -118,6 +119,7 @@ def bench_decode(llm, batch: int, context: int, steps: int, warmup: int, seed: i
     e0.record()
     for _ in range(steps):
         eng.step()
+    eng.drain()                                                      # and nothing when it stops: K steps queued, K read
     e1.record()
     sync()
     dt = time.perf_counter() - t0
@@ -149,6 +151,7 @@ def bench_generate(llm, batch: int, prompt_len: int, new_tokens: int, seed: int)
             for p in random_prompts(batch, prompt_len, cfg.vocab_size, seed)]
     while any(r.num_computed < r.prompt_len for r in reqs):
         eng.step()
+    eng.drain()
     sync()                                                  # every request has its first token; all decode from here
     assert all(not r.done for r in reqs) and len(eng.scheduler.running) == batch
     steps = new_tokens - max(r.num_generated for r in reqs)
@@ -159,6 +162,7 @@ def bench_generate(llm, batch: int, prompt_len: int, new_tokens: int, seed: int)
     e0.record()
     for _ in range(steps):
         eng.step()
+    eng.drain()
     e1.record()
     sync()
     dt = time.perf_counter() - t0
@@ -182,9 +186,10 @@ def profile_decode_step(llm, batch: int, context: int, seed: int) -> dict:
             for p in random_prompts(batch, prompt_len, cfg.vocab_size, seed)]
     while any(r.num_computed < r.prompt_len for r in reqs):
         eng.step()
-    graph_runner, eager = eng.runner, ModelRunner(llm.model, llm.cache)
+    eng.drain()
+    graph_runner, eager, overlap = eng.runner, ModelRunner(llm.model, llm.cache), eng.overlap
     eager.fit_context = graph_runner.fit_context
-    eng.runner = eager
+    eng.runner, eng.overlap = eager, False                   # one step at a time, read before the next
     try:
         for _ in range(3):
             eng.step()
@@ -192,7 +197,7 @@ def profile_decode_step(llm, batch: int, context: int, seed: int) -> dict:
         with timer.measuring():
             eng.step()
     finally:
-        eng.runner = graph_runner
+        eng.runner, eng.overlap = graph_runner, overlap
     for r in reqs:
         eng.abort(r)
     return timer.summary()
@@ -308,6 +313,7 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--no-overlap", action="store_true", help="read every decode step's tokens before queueing the next")
     ap.add_argument("--no-fp32", action="store_true", help="skip the 32-bit point")
     ap.add_argument("--fp32-layers", type=int, default=4, help="layers of the model the 32-bit point runs")
     ap.add_argument("--profile", action="store_true", help="add the time of one eager decode step by class of kernel")
@@ -339,7 +345,7 @@ def main() -> int:
     llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
               num_blocks=max_batch * (-(-max_len // page)) + 8, max_num_seqs=max_batch, max_batched_tokens=2048,
               max_model_len=max_len, graphs=not args.no_graphs, graph_warmup_tokens=0, prefix_caching=False,
-              tune_library=not args.no_tune)
+              tune_library=not args.no_tune, overlap=not args.no_overlap)
     elem = 2 if args.dtype in ("bfloat16", "bf16") else 4
     dtype_key = "bfloat16" if elem == 2 else "float32"
 
@@ -407,6 +413,7 @@ def main() -> int:
             "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "page_size": page,
             "prefill_tokens": args.prefill_tokens, "graphs": not args.no_graphs, "library_tuning": not args.no_tune, "sampling": "greedy",
+            "overlap": not args.no_overlap,
             "decode_graph_replays": main_run["graph_replays"], "mean_context": round(main_run["mean_context"], 1),
         },
         "prefill": {"value": round(pre["tok_s"], 1), "tokens": args.prefill_tokens, "ms": round(pre["s"] * 1e3, 3),

@@ -3,7 +3,7 @@
 Options keep the names and meanings of the reference's launcher where it has them
 (tensorline/server.py:256-283): ``--model`` (default from ``TL_MODEL``), ``--device``, ``--dtype``,
 ``--max-num-seqs``, ``--max-batched-tokens``, ``--num-blocks``, ``--no-cuda-graphs``,
-``--graph-warmup-tokens``, ``--no-prefix-caching``, ``--kv-cache-gb``.  Its server, engine choice,
+``--graph-warmup-tokens``, ``--no-prefix-caching``, ``--no-overlap``, ``--kv-cache-gb``.  Its server, engine choice,
 speculation, overlap, quantisation and multi-model options have no counterpart here.  Added: the
 constructor-only options of the reference (``--block-size``, ``--max-model-len``) and the request
 options (``--max-tokens``, ``--temperature``, ``--top-p``, ``--seed``).
@@ -31,6 +31,7 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--graph-warmup-tokens", type=int, default=512,
                     help="capture the decode graphs before serving (0 = at first use)")
     ap.add_argument("--no-prefix-caching", action="store_true", help="never reuse KV pages across requests")
+    ap.add_argument("--no-overlap", action="store_true", help="read every decode step's tokens before queueing the next step")
     ap.add_argument("--tune-library", action="store_true",
                     help="at start-up, let the library pick its kernels for full prompt portions by measurement")
 
@@ -42,7 +43,7 @@ def _make_llm(a):
     return LLM(a.model, device=a.device, dtype=a.dtype, max_num_seqs=a.max_num_seqs,
                max_batched_tokens=a.max_batched_tokens, num_blocks=a.num_blocks, kv_cache_gb=a.kv_cache_gb,
                block_size=a.block_size, max_model_len=a.max_model_len, graphs=not a.no_graphs,
-               graph_warmup_tokens=a.graph_warmup_tokens, prefix_caching=not a.no_prefix_caching,
+               graph_warmup_tokens=a.graph_warmup_tokens, prefix_caching=not a.no_prefix_caching, overlap=not a.no_overlap,
                tune_library=a.tune_library)
 
 

@@ -18,6 +18,7 @@ class EngineConfig:
     graphs: bool = True                  # replay pure-decode steps from a HIP graph (--no-cuda-graphs there)
     graph_warmup_tokens: int = 512       # capture graphs for contexts up to this many tokens at start-up
     prefix_caching: bool = True
+    overlap: bool = True                 # queue decode step t + 1 before reading step t's tokens (--no-overlap there)
     tune_library: bool = False           # at start-up, let the library pick its kernels for full prompt portions by measurement
     device: str = "cuda:0"
 

@@ -181,9 +181,9 @@ class GraphRunner(ModelRunner):
 
     # ---- one step ------------------------------------------------------------------------------
     @torch.inference_mode()
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], token_source: torch.Tensor | None = None) -> torch.Tensor:
         if not self.can_run(entries):
-            return super().step(entries)
+            return super().step(entries, token_source)
         n = len(entries)
         B, C = self._bucket(n), self._context_bucket(max(e.start for e in entries) + 1)
         cap = self.graphs.get((B, C)) or self._capture(B, C)
@@ -199,6 +199,8 @@ class GraphRunner(ModelRunner):
             cap.starts = np.fromiter((e.start for e in entries), np.int64, n)
         # The copy is queued, not awaited: copy and graph reach the GPU back to back.
         cap.dev.copy_(cap.host, non_blocking=True)
+        if token_source is not None:
+            self._take_tokens(cap.dev, cap.packed, token_source)
         if cap.copied is None:
             cap.copied = torch.cuda.Event()
         cap.copied.record()

@@ -71,7 +71,7 @@ class LLM:
                 runner.warmup(min(ec.graph_warmup_tokens, ec.max_model_len))
         self.engine = InferenceEngine(self.model, self.cache, max_num_seqs=ec.max_num_seqs,
                                       max_batched_tokens=ec.max_batched_tokens, max_model_len=ec.max_model_len,
-                                      default_stops=set(self.model.spec.eos_token_ids), runner=runner)
+                                      default_stops=set(self.model.spec.eos_token_ids), runner=runner, overlap=ec.overlap)
         # with or without graphs, every step makes the choices that depend on the longest context alike
         self.engine.runner.fit_context = -(-ec.max_model_len // ec.block_size) * ec.block_size
 

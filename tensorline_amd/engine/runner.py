@@ -88,11 +88,23 @@ class ModelRunner:
         return ctx, views
 
     # ---- one step ------------------------------------------------------------------------
+    @staticmethod
+    def _take_tokens(dev: torch.Tensor, packed: PackedBatch, token_source: torch.Tensor) -> None:
+        """Overwrite the step's token ids on the device with ``token_source`` (int32, a token per
+        entry in the order of the entries): the step then runs on tokens the host has not seen yet."""
+        if packed.T != packed.S:
+            raise ValueError("tokens can be taken from the device only for steps of one token per request")
+        off, _ = packed.offsets["ids"]
+        n = token_source.numel()
+        dev[off:off + n].copy_(token_source, non_blocking=True)
+
     @torch.inference_mode()
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Logits [number of wanted places, vocab] in float32."""
+    def step(self, entries: Sequence[StepEntry], token_source: torch.Tensor | None = None) -> torch.Tensor:
+        """Logits [number of wanted places, vocab] in float32.  ``token_source``: see ``_take_tokens``."""
         packed = self.pack(entries)
         dev = self._upload(packed.data)
+        if token_source is not None:
+            self._take_tokens(dev, packed, token_source)
         ctx, views = self.context(packed, dev)
         self.steps += 1
         return self.model.forward(ctx, views)

@@ -31,16 +31,22 @@ class Sampler:
     def __init__(self, device):
         self.device = device
 
-    def sample(self, logits: torch.Tensor, temperatures: list[float], top_ps: list[float],
-               seeds: list[int], indices: list[int]) -> list[int]:
-        """One token per row of float32 ``logits`` [R, V]."""
+    def sample_device(self, logits: torch.Tensor, temperatures: list[float], top_ps: list[float],
+                      seeds: list[int], indices: list[int]) -> torch.Tensor:
+        """One token per row of float32 ``logits`` [R, V], as an int32 tensor on the device: nothing
+        is awaited, so the caller may queue more work before it looks at the tokens."""
         R = logits.shape[0]
         if R == 0:
-            return []
+            return torch.empty(0, dtype=torch.int32, device=logits.device)
         if all(t <= 0 for t in temperatures):
-            return kernels.argmax(logits).tolist()
+            return kernels.argmax(logits)
         u = [uniform_for(s, i) for s, i in zip(seeds, indices)]
         params = torch.tensor([temperatures, top_ps, u], dtype=torch.float32).to(self.device)
         return kernels.sample(logits, params[0], params[1], params[2],
                               any_top_p=any(p < 1.0 for p in top_ps),
-                              any_greedy=any(t <= 0 for t in temperatures)).tolist()
+                              any_greedy=any(t <= 0 for t in temperatures))
+
+    def sample(self, logits: torch.Tensor, temperatures: list[float], top_ps: list[float],
+               seeds: list[int], indices: list[int]) -> list[int]:
+        """The same, awaited and as a list."""
+        return self.sample_device(logits, temperatures, top_ps, seeds, indices).tolist()

@@ -234,3 +234,53 @@ def test_engine_reports_distributions_of_latency_and_batch_size(tiny, cpu_kernel
     bs = c["batch_size"]
     assert bs["count"] == c["steps"] and bs["max"] == 3 == c["max_running_seen"]
     assert sum(bs["buckets"].values()) == bs["count"] and bs["buckets"]["le_4"] > 0
+
+
+def test_decode_steps_overlap_and_change_no_token(tiny, cpu_kernels):
+    """Steady decoding queues step t + 1 before it reads step t's tokens (they are taken from the
+    device): the tokens are those of the plain implementation with the overlap on and off, for
+    every small token limit (the last token of a request is never run ahead of), and a request
+    that a stop token ends while the next step is in flight costs its neighbours nothing."""
+    d, prompts, want = tiny
+    for overlap in (True, False):
+        eng = make_engine(d, overlap=overlap)
+        reqs = [eng.add_request(prompts[i], SamplingParams(17, stop_token_ids=NO_STOP)) for i in (1, 3, 5)]
+        eng.run_until_done()
+        assert [r.output_tokens for r in reqs] == [want[(i, 17)] for i in (1, 3, 5)]
+        c = eng.counters()
+        assert (c["overlapped_steps"] > 10) == overlap and c["tokens_generated"] == 3 * 17 and eng.cache.all_free()
+    for limit in (1, 2, 3, 4):
+        eng = make_engine(d)
+        reqs = [eng.add_request(prompts[i], SamplingParams(limit + k, stop_token_ids=NO_STOP)) for k, i in enumerate((1, 3))]
+        eng.run_until_done()
+        assert [r.output_tokens for r in reqs] == [want[(1, 17)][:limit], want[(3, 17)][:limit + 1]]
+        assert all(r.stats.finish_reason == "length" for r in reqs) and eng.cache.all_free()
+    # a stop token in the middle: the request ends there, the other goes on to its limit
+    full = want[(1, 17)]
+    stop = full[6]
+    eng = make_engine(d)
+    a = eng.add_request(prompts[1], SamplingParams(17, stop_token_ids={stop}))
+    b = eng.add_request(prompts[3], SamplingParams(17, stop_token_ids=NO_STOP))
+    eng.run_until_done()
+    assert a.output_tokens == full[:full.index(stop)] and a.stats.finish_reason == "stop"
+    assert b.output_tokens == want[(3, 17)] and eng.counters()["overlapped_steps"] > 0 and eng.cache.all_free()
+    # the longest length the engine allows ends a request as a token limit does
+    eng = make_engine(d, max_model_len=len(prompts[3]) + 5)
+    r = eng.add_request(prompts[3], SamplingParams(500, stop_token_ids=NO_STOP))
+    eng.run_until_done()
+    assert r.output_tokens == want[(3, 17)][:5] and r.stats.finish_reason == "length"
+
+
+def test_abort_while_a_step_is_in_flight(tiny, cpu_kernels):
+    d, prompts, want = tiny
+    eng = make_engine(d)
+    a = eng.add_request(prompts[1], SamplingParams(17, stop_token_ids=NO_STOP))
+    b = eng.add_request(prompts[3], SamplingParams(17, stop_token_ids=NO_STOP))
+    for _ in range(6):
+        eng.step()
+    assert eng._inflight is not None                      # a decode step is queued and unread
+    eng.abort(a)
+    eng.run_until_done()
+    assert a.stats.finish_reason == "abort" and a.output_tokens == want[(1, 17)][:len(a.output_tokens)]
+    assert b.output_tokens == want[(3, 17)] and eng.cache.all_free()
+    assert eng.drain() == []
