@@ -11,7 +11,9 @@ roofline, and under ``points`` decode throughput at batch 1 and 64 at the same c
 (``decode_b*``) and the decode phase of the workload the shape is quoted with, 2,048-token
 prompts and 256 generated tokens each, at batch 1, 8 and 64 (``gen_b*``), each with its time per
 step, its mean context and its share of the HBM roofline.  ``fp32`` holds the cost of the true
-32-bit path at the same layer sizes with fewer layers (both numbers are named).  The fractions
+32-bit path at the same layer sizes with fewer layers (both numbers are named), ``sizes`` batch 8
+decoding and the same prefill at the 14B and 32B shapes (all layers) and, for the default shape,
+batch 8 decoding at a context of 32,768 and a prompt portion behind 30,720 cached tokens.  The fractions
 are of the published peaks; ``machine`` holds what this GPU reaches on a plain copy and on a
 large library product, and the ``frac_of_measured_*`` fields are the same figures relative to
 those.  ``--profile`` adds the time of one eagerly run decode step by class of kernel.
@@ -19,6 +21,7 @@ those.  ``--profile`` adds the time of one eagerly run decode step by class of k
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -226,6 +229,40 @@ def bench_prefill(llm, tokens: int, reps: int, seed: int) -> dict:
     return {"s": best, "tok_s": tokens / best}
 
 
+def prefill_portion_flops(cfg, tokens: int, context: int) -> float:
+    """A portion of ``tokens`` tokens behind ``context`` cached ones, logits for its last position."""
+    L, V, H = cfg.num_hidden_layers, cfg.vocab_size, cfg.hidden_size
+    linear = 2.0 * tokens * L * layer_matrix_params(cfg)
+    attn = 4.0 * cfg.num_attention_heads * cfg.head_dim * (tokens * context + tokens * (tokens + 1) / 2) * L
+    return linear + attn + 2.0 * V * H
+
+
+def bench_prefill_portion(llm, context: int, tokens: int, reps: int, seed: int) -> dict:
+    """A prompt portion of ``tokens`` tokens in one step behind ``context`` tokens that earlier steps
+    cached (in portions of the same size), logits for its last position."""
+    from tensorline_amd.engine.batch import StepEntry
+    from tensorline_amd.ops import kernels
+    cfg, cache, runner = llm.model_config, llm.cache, llm.engine.runner
+    prompt = random_prompts(1, context + tokens, cfg.vocab_size, seed)[0]
+    rid = ("portion", 0)
+    cache.add_request(rid)
+    assert cache.grow(rid, context + tokens)
+    for start in range(0, context, tokens):
+        n = min(tokens, context - start)
+        runner.step([StepEntry(rid, prompt[start:start + n], start, [])])
+    times = []
+    for _ in range(reps + 1):                                          # the same portion again: it overwrites its own keys
+        sync()
+        t0 = time.perf_counter()
+        logits = runner.step([StepEntry(rid, prompt[context:], context, [tokens - 1])])
+        kernels.argmax(logits).tolist()
+        sync()
+        times.append(time.perf_counter() - t0)
+    cache.release(rid)
+    best = min(times[1:])
+    return {"s": best, "tok_s": tokens / best}
+
+
 def measure_machine(dtype) -> dict:
     """What this GPU reaches on two plain jobs, beside the published peaks: a device-to-device
     copy of 2 GiB (bytes read plus bytes written per second) and a square library product of
@@ -315,6 +352,7 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-overlap", action="store_true", help="read every decode step's tokens before queueing the next")
     ap.add_argument("--no-fp32", action="store_true", help="skip the 32-bit point")
+    ap.add_argument("--no-sizes", action="store_true", help="skip the 14B and 32B shapes and the 32k contexts")
     ap.add_argument("--fp32-layers", type=int, default=4, help="layers of the model the 32-bit point runs")
     ap.add_argument("--profile", action="store_true", help="add the time of one eager decode step by class of kernel")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's heuristic choice of kernels for prompt portions")
@@ -375,7 +413,8 @@ def main() -> int:
     fp32 = None
     if elem == 2 and not args.no_points and not args.no_fp32:
         # the true 32-bit path at the same layer sizes, fewer layers: what the equality checks cost
-        del llm
+        llm = None
+        gc.collect()
         torch.cuda.empty_cache()
         cfg32 = make_config(args.fp32_layers, args.shape)
         llm32 = LLM(config=cfg32, seed=args.seed, dtype="float32", device="cuda:0", block_size=page,
@@ -389,6 +428,45 @@ def main() -> int:
                 "decode_b8_tok_s": dec32["tok_s"], "decode_b8_ms": dec32["ms"], "decode_b8_ctx": dec32["ctx"],
                 "decode_b8_hbm_frac": dec32["hbm_frac"]}
         del llm32
+    sizes = None
+    if elem == 2 and not args.no_points and not args.no_sizes and args.shape == "7b" and not args.layers:
+        # further sizes and contexts, all layers of each shape: batch 8 decoding at the same context and the
+        # same prefill for the 14B and 32B shapes; for the default shape batch 8 decoding at a context of
+        # 32,768 and a prompt portion behind 30,720 cached tokens
+        llm = None
+        gc.collect()
+        torch.cuda.empty_cache()
+        sizes = {}
+
+        def other(shape: str, context: int, batch: int, steps: int):
+            c = make_config(0, shape)
+            length = context + 16
+            m = LLM(config=c, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
+                    num_blocks=batch * (-(-length // page)) + 8, max_num_seqs=batch, max_batched_tokens=2048,
+                    max_model_len=length, graphs=not args.no_graphs, graph_warmup_tokens=0, prefix_caching=False,
+                    tune_library=not args.no_tune, overlap=not args.no_overlap)
+            dec = with_roofline(bench_decode(m, batch, context, steps, 4, args.seed + 11), batch, c)
+            return c, m, {"layers": c.num_hidden_layers, f"decode_b{batch}_tok_s": dec["tok_s"], f"decode_b{batch}_ms": dec["ms"],
+                          f"decode_b{batch}_ctx": dec["ctx"], f"decode_b{batch}_hbm_frac": dec["hbm_frac"]}
+        for shape in ("14b", "32b"):
+            c, m, out = other(shape, args.context, 8, 16)
+            p2 = bench_prefill(m, args.prefill_tokens, 2, args.seed + 2)
+            out.update({"prefill_tok_s": round(p2["tok_s"], 1), "prefill_ms": round(p2["s"] * 1e3, 3),
+                        "prefill_frac": round(prefill_flops(c, args.prefill_tokens) / p2["s"] / PEAK_FLOPS[dtype_key], 4)})
+            sizes[shape] = out
+            del m
+            gc.collect()
+            torch.cuda.empty_cache()
+        c, m, out = other("7b", 32768, 8, 16)
+        behind = 32768 - args.prefill_tokens
+        p3 = bench_prefill_portion(m, behind, args.prefill_tokens, 2, args.seed + 2)
+        out.update({"portion_behind": behind, "portion_tokens": args.prefill_tokens, "portion_tok_s": round(p3["tok_s"], 1),
+                    "portion_ms": round(p3["s"] * 1e3, 3),
+                    "portion_frac": round(prefill_portion_flops(c, args.prefill_tokens, behind) / p3["s"] / PEAK_FLOPS[dtype_key], 4)})
+        sizes["7b_32k"] = out
+        del m
+        gc.collect()
+        torch.cuda.empty_cache()
     step_s = main_run["ms_per_step"] / 1e3
     achieved = decode_bytes(cfg, args.batch, int(main_run["mean_context"]), elem) / step_s / 1e9
     flops = prefill_flops(cfg, args.prefill_tokens)
@@ -427,6 +505,8 @@ def main() -> int:
     }
     if fp32 is not None:
         line["fp32"] = fp32
+    if sizes is not None:
+        line["sizes"] = sizes
     if profile is not None:
         line["profile"] = profile
     print(json.dumps(line))
