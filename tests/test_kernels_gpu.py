@@ -421,14 +421,17 @@ def test_attention_decode_long_contexts(lens, split):
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("bs", [8, 16, 64, 128, 24])
-def test_attention_prompt_tiles_page_sizes_and_long_tables(bs):
+@pytest.mark.parametrize("d,bs", [(128, 8), (128, 16), (128, 32), (128, 64), (128, 128), (128, 24), (64, 8), (64, 16),
+                                  (64, 32), (64, 64), (32, 16), (32, 32), (32, 64), (32, 256)])
+def test_attention_prompt_tiles_page_sizes_and_long_tables(d, bs):
     """Prompt portions on the kernel that stages 64-key tiles in LDS: pages smaller than, equal to
     and larger than a tile, a page table of more than 512 entries (8 and 16-token pages), a far key
     that dominates, a portion that starts and ends inside a tile, a short sequence beside it.  Pages
-    of 24 tokens (no power of two) take the independent-wave kernel instead."""
+    of 24 tokens (no power of two) take the independent-wave kernel instead.  Where the 64 units of
+    each of a wave's loads lie in one page (head size x page size >= 2048) the loader works with one
+    page id per load, and the values' tile in LDS is cut by pages; elsewhere with one per lane."""
     lens, q_lens = [9000, 131, 70], [300, 131, 3]
-    got, want = _attention_case(torch.bfloat16, 28, 4, 128, bs, lens, q_lens, spike=True, seed=bs, path="mfma")
+    got, want = _attention_case(torch.bfloat16, 28, 4, d, bs, lens, q_lens, spike=True, seed=bs, path="mfma")
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
 
 
