@@ -80,7 +80,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
     T* __restrict__ out, int out_stride, int tiles_per_seq, int QT, int GC, int nq, int nkv, int bs, int KT,
-    int window, float scale) {
+    int window, float scale, int nsplit, int split_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
     constexpr int d = DB * 16;
     extern __shared__ float smem[];
     constexpr int ks_ld = d + 4;
@@ -96,7 +96,8 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     const int s = blockIdx.x / tiles_per_seq, ti = blockIdx.x - s * tiles_per_seq;
     const int kvh = blockIdx.y;
     const int G = nq / nkv;
-    const int g0 = blockIdx.z * GC;                       // first query head of this chunk within the group
+    const int chunk = blockIdx.z / nsplit, sp = blockIdx.z - chunk * nsplit;
+    const int g0 = chunk * GC;                            // first query head of this chunk within the group
     const int gc = (G - g0 < GC) ? G - g0 : GC;
     const int t_first = q_start[s] + ti * QT, t_end = q_start[s + 1];
     if (t_first >= t_end) return;
@@ -238,13 +239,20 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
         }
     };
 
-    const int k_first = (k_lo / KT) * KT;
+    // With split keys this work-group walks the tiles of split sp only: keys [sp * split_keys,
+    // (sp + 1) * split_keys), a multiple of KT at absolute positions, so that the same keys are summed
+    // together whatever the context length and the number of splits of the launch.
+    int k_first = (k_lo / KT) * KT, k_end = k_hi;
+    if (nsplit > 1) {
+        k_first = (k_first > sp * split_keys) ? k_first : sp * split_keys;
+        k_end = (k_end < (sp + 1) * split_keys) ? k_end : (sp + 1) * split_keys;
+    }
     const int key_blocks = KT / 16;
-    fetch(k_first);
-    for (int k0 = k_first; k0 < k_hi; k0 += KT) {
+    if (k_first < k_end) fetch(k_first);
+    for (int k0 = k_first; k0 < k_end; k0 += KT) {
         to_lds(k0);
         __syncthreads();
-        if (k0 + KT < k_hi) fetch(k0 + KT);
+        if (k0 + KT < k_end) fetch(k0 + KT);
 
         if (k0 < w_hi && k0 + KT > w_lo) {                 // a tile none of the wave's rows sees is skipped
             // ---- S = Q K^T: per block of 16 keys, 4 DB products; lane holds rows 4 lg + v, key li ----
@@ -320,6 +328,24 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     }
 
     // this lane holds output rows 4 lg + v at head dimensions 16 db + li
+    if (nsplit > 1) {
+        // the split's sums as they are, with their maximum and denominator (a split that holds no key
+        // of a row leaves -inf, 0 and zeros); attn_generic_merge_kernel puts the splits together
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            if (my_pos[v] < 0) continue;
+            const int row = wave * AG_WROWS + 4 * lg + v;
+            const int i = row / GC, g = row - i * GC;
+            const size_t part = ((size_t)(t_first + i) * nq + (kvh * G + g0 + g)) * nsplit + sp;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) ws_o[part * d + db * 16 + li] = acc[db][v];
+            if (li == 0) {
+                ws_ml[part * 2] = m[v];
+                ws_ml[part * 2 + 1] = l[v];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
         if (my_pos[v] < 0) continue;
@@ -332,16 +358,47 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     }
 }
 
+// out[t, h, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(m_s - max m), over the splits in
+// ascending order (a split without keys of the row has l_s = 0 and is left out).  One work-group
+// per (row, head), a thread per head dimension.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_generic_merge_kernel(const float* __restrict__ ws_o,
+                                                                 const float* __restrict__ ws_ml, T* __restrict__ out,
+                                                                 int out_stride, int nq, int d, int nsplit) {
+    const int t = blockIdx.x, h = blockIdx.y, dd = threadIdx.x;
+    if (dd >= d) return;
+    const size_t base = ((size_t)t * nq + h) * nsplit;
+    float M = -INFINITY;
+    for (int s = 0; s < nsplit; ++s)
+        if (ws_ml[(base + s) * 2 + 1] > 0.f) M = fmaxf(M, ws_ml[(base + s) * 2]);
+    float num = 0.f, den = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < nsplit; ++s) {
+        const float ls = ws_ml[(base + s) * 2 + 1];
+        if (ls > 0.f) {
+            const float w = expf(ws_ml[(base + s) * 2] - M);
+            num += w * ws_o[(base + s) * d + dd];
+            den += w * ls;
+        }
+    }
+    out[(size_t)t * out_stride + (size_t)h * d + dd] = tl_from_float<T>(den > 0.f ? num / den : 0.f);
+}
+
 static size_t ag_lds_bytes(int d, int KT) {
     return sizeof(float) * ((size_t)KT * (d + 4) + (size_t)d * (KT + 4) + 4 * AG_WROWS * (KT + 4)) + sizeof(int) * (2 * AG_ROWS);
 }
 
 // q_start: int32 [S + 1], the first row of each sequence in the flat batch (rows of a sequence are
-// consecutive); max_query_len: the most tokens one sequence brings to this step.
+// consecutive); max_query_len: the most tokens one sequence brings to this step.  nsplit > 1 cuts
+// the keys into runs of split_keys (a multiple of 64) at absolute positions, one work-group each,
+// and a second kernel merges them: for steps of few tokens with long contexts, which would
+// otherwise be walked by one work-group per sequence and key/value head.  nsplit * split_keys must
+// cover the longest context; ws holds T * nq * nsplit * (d + 2) floats.
 extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                     const int32_t* tables, int NB, const int32_t* q_start, const int32_t* pos,
                                     void* out, int out_stride, int dtype, int T, int S, int max_query_len, int nq, int nkv,
-                                    int d, int bs, int window, float scale, hipStream_t stream) {
+                                    int d, int bs, int window, float scale, int nsplit, int split_keys, float* ws,
+                                    hipStream_t stream) {
     TL_CHECK_ARG(T >= 0 && S >= 0 && nq > 0 && nkv > 0 && d > 0 && bs > 0 && NB > 0,
                  "tl_attention_generic: bad sizes T=%d S=%d nq=%d nkv=%d d=%d page=%d NB=%d", T, S, nq, nkv, d, bs, NB);
     TL_CHECK_ARG(nq % nkv == 0, "tl_attention_generic: %d query heads are not a multiple of %d key/value heads", nq, nkv);
@@ -354,7 +411,12 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
     const int GC = (G < AG_ROWS) ? G : AG_ROWS;           // query heads per work-group
     const int QT = AG_ROWS / GC;                          // tokens per work-group
     const int chunks = tl_ceil_div(G, GC);
-    TL_CHECK_ARG(chunks <= 65535, "tl_attention_generic: group of %d query heads is too large", G);
+    TL_CHECK_ARG(nsplit >= 1 && (long long)chunks * nsplit <= 65535,
+                 "tl_attention_generic: %d chunks of query heads x %d key splits are more than a launch takes", chunks, nsplit);
+    TL_CHECK_ARG(nsplit == 1 || (ws && split_keys > 0 && split_keys % 64 == 0),
+                 "tl_attention_generic: split keys need a workspace and a split length that is a multiple of 64 (%d)", split_keys);
+    float* ws_o = ws;
+    float* ws_ml = ws ? ws + (size_t)T * nq * nsplit * d : nullptr;
     const int tiles_per_seq = tl_ceil_div(max_query_len, QT);
     const long long groups = (long long)S * tiles_per_seq;
     TL_CHECK_ARG(groups <= 0x7fffffffLL, "tl_attention_generic: too many work-groups");
@@ -362,11 +424,11 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
     const size_t smem = ag_lds_bytes(d, KT);
     TL_CHECK_ARG(smem <= 160 * 1024, "tl_attention_generic: head size %d needs %zu bytes of LDS", d, smem);
     TL_CHECK_ARG(KT * d / 4 <= AG_MAXC * AG_THREADS, "tl_attention_generic: a tile of head size %d has too many pieces", d);
-    dim3 grid((unsigned)groups, nkv, chunks), block(AG_THREADS);
+    dim3 grid((unsigned)groups, nkv, chunks * nsplit), block(AG_THREADS);
 #define AG_LAUNCH(TT, DB)                                                                                             \
     hipLaunchKernelGGL((attn_generic_kernel<TT, DB>), grid, block, smem, stream, (const TT*)q, q_stride,              \
                        (const TT*)k_cache, (const TT*)v_cache, tables, NB, q_start, pos, (TT*)out, out_stride,          \
-                       tiles_per_seq, QT, GC, nq, nkv, bs, KT, window, scale)
+                       tiles_per_seq, QT, GC, nq, nkv, bs, KT, window, scale, nsplit, split_keys, ws_o, ws_ml)
 #define AG_CASE(TT, DB) \
     case DB: AG_LAUNCH(TT, DB); break;
 #define AG_DISPATCH(TT)                                                                              \
@@ -386,5 +448,15 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
 #undef AG_CASE
 #undef AG_LAUNCH
     TL_CHECK_LAUNCH("tl_attention_generic");
+    if (nsplit > 1) {
+        dim3 mgrid(T, nq);
+        if (dtype == TL_F32)
+            hipLaunchKernelGGL(attn_generic_merge_kernel<float>, mgrid, dim3(256), 0, stream, ws_o, ws_ml, (float*)out,
+                               out_stride, nq, d, nsplit);
+        else
+            hipLaunchKernelGGL(attn_generic_merge_kernel<bf16_t>, mgrid, dim3(256), 0, stream, ws_o, ws_ml, (bf16_t*)out,
+                               out_stride, nq, d, nsplit);
+        TL_CHECK_LAUNCH("tl_attention_generic merge");
+    }
     return 0;
 }

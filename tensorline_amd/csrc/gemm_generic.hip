@@ -8,10 +8,12 @@
 // One output element is summed over k in one fixed order: steps of 16 from k = 0 upwards, four
 // products per step, the lanes' k within a step fixed by the operand layout.  The order does not
 // depend on M or on which tile shape the launch picked, so cutting a batch differently does not
-// change a bit of a result, and neither does the number of rows that come along.
+// change a bit of a result, and neither does the number of rows that come along (from 17 rows on;
+// up to 16 rows have an order of their own, see gemm_fewrows_kernel).
 //
 // Tiles: four waves compute BM x BN outputs, a wave MB x NB blocks of 16 x 16; 128 x 128 for many
-// rows, 64 x 128 and 32 x 64 for few (more work-groups stream the weights then).  A k-step's rows
+// rows, 64 x 128 and 32 x 64 for few (more work-groups stream the weights then); at most 16 rows
+// have a kernel of their own (gemm_fewrows_kernel), which sums K in segments.  A k-step's rows
 // of A and W go from memory into registers while the step before is computed, then as float into
 // LDS [row][16 + 4] (the padding keeps the 16-byte operand reads off each other's banks).
 //
@@ -57,6 +59,21 @@ __device__ __forceinline__ float4 gg_load4<bf16_t>(const bf16_t* __restrict__ ba
     r.z = (k + 2 < K) ? tl_to_float(base[k + 2]) : 0.f;
     r.w = (k + 3 < K) ? tl_to_float(base[k + 3]) : 0.f;
     return r;
+}
+
+// The same four k with nothing to check: the caller knows that the row exists, that all four k do
+// and that the piece is aligned.
+template <typename T>
+__device__ __forceinline__ float4 gg_load4_whole(const T* __restrict__ p);
+template <>
+__device__ __forceinline__ float4 gg_load4_whole<float>(const float* __restrict__ p) {
+    return *reinterpret_cast<const float4*>(p);
+}
+template <>
+__device__ __forceinline__ float4 gg_load4_whole<bf16_t>(const bf16_t* __restrict__ p) {
+    const uint2 raw = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                       __uint_as_float(raw.y & 0xffff0000u));
 }
 
 // WM x WN waves (WM * WN == 4), each MB x NB blocks of 16 x 16.
@@ -156,6 +173,96 @@ __global__ __launch_bounds__(GG_THREADS) void gemm_generic_kernel(const TA* __re
     }
 }
 
+// At most 16 rows (a decode step of few sequences): the work is streaming W once, and a tile of the
+// kernel above would leave most of the GPU without work (56 work-groups for 3,584 columns) with one
+// k-step in flight each.  Here a work-group owns 16 columns and its waves share K: K is cut into
+// segments of GF_SEG at absolute k, wave w sums segments w, w + waves, ... each in the order above
+// (steps of 16 upwards, four products per step), with the next GF_RING - 1 steps' operands on their
+// way in a ring of registers, and the segments' sums are added in ascending order at the end.  So
+// one output element is again summed in one fixed order that depends on K alone, not on M (1 to 16),
+// on the number of waves or on timing; it is not the order of the kernel above, whose results differ
+// from this one's by rounding.
+#define GF_SEG 512
+#ifndef GF_RING
+#define GF_RING 4
+#endif
+#ifndef GF_WAVES
+#define GF_WAVES 8
+#endif
+#define GF_MAX_SEGMENTS 64    // 64 KB of LDS for the segments' sums: K up to 32,768 (beyond: the kernel above)
+
+template <typename TA, typename TW, typename TO>
+__global__ __launch_bounds__(512) void gemm_fewrows_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
+                                                           const float* __restrict__ bias, TO* __restrict__ C, int M,
+                                                           int N, int K, int lda, int ldc, int a_vec, int w_vec) {
+    extern __shared__ float gf_part[];                       // [segment][register v][lane]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int li = lane & 15, lg = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int nseg = (K + GF_SEG - 1) / GF_SEG;
+    constexpr int SPS = GF_SEG / GG_KS;                      // steps per segment
+    const TW* wrow = W + (size_t)(n0 + li) * K;
+    const TA* arow = A + (size_t)li * lda;
+    const bool w_ok = n0 + li < N, a_ok = li < M;
+    // Whole steps (all 16 k inside K, aligned pieces) load without a condition, so that the loads of
+    // the steps ahead stay in flight: a row that does not exist is read from one that does (what it
+    // brings only reaches outputs that are not written).
+    const TW* wrow_any = W + (size_t)(w_ok ? n0 + li : N - 1) * K;
+    const TA* arow_any = A + (size_t)(a_ok ? li : 0) * lda;
+    const bool pieces_whole = a_vec != 0 && w_vec != 0;
+    auto load_step = [&](int k0, float4& wv, float4& av) {
+        if (pieces_whole && k0 + GG_KS <= K) {                  // the same for the whole wave
+            wv = gg_load4_whole<TW>(wrow_any + k0 + 4 * lg);
+            av = gg_load4_whole<TA>(arow_any + k0 + 4 * lg);
+        } else {                                              // past K (the last segment's end): zeros
+            wv = gg_load4<TW>(wrow, w_ok, k0 + 4 * lg, K, w_vec != 0);
+            av = gg_load4<TA>(arow, a_ok, k0 + 4 * lg, K, a_vec != 0);
+        }
+    };
+    // this wave's steps, numbered through its segments: step j is step j % SPS of segment wave + (j / SPS) * nwaves
+    const int my_segs = (nseg - wave + nwaves - 1) / nwaves;   // 0 for a wave beyond the segments
+    const int nsteps = my_segs * SPS;
+    auto k_of = [&](int j) { return (wave + (j / SPS) * nwaves) * GF_SEG + (j % SPS) * GG_KS; };
+    float4 wreg[GF_RING], areg[GF_RING];
+#pragma unroll
+    for (int r = 0; r < GF_RING - 1; ++r) {
+        if (r < nsteps) load_step(k_of(r), wreg[r], areg[r]);
+    }
+    gg_f32x4 acc = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int jb = 0; jb < nsteps; jb += GF_RING) {
+#pragma unroll
+        for (int r = 0; r < GF_RING; ++r) {
+            const int j = jb + r;
+            if (j < nsteps) {                                 // the same for the whole wave
+                const int ahead = j + GF_RING - 1;
+                if (ahead < nsteps) load_step(k_of(ahead), wreg[(r + GF_RING - 1) % GF_RING], areg[(r + GF_RING - 1) % GF_RING]);
+                // as in the kernel above: the lane gives row li of A and row li of the W tile at k = k0 + 4 lg + v
+                // to the v-th product and holds C[4 lg + v][n0 + li]
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[r].x, wreg[r].x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[r].y, wreg[r].y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[r].z, wreg[r].z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(areg[r].w, wreg[r].w, acc, 0, 0, 0);
+                if (j % SPS == SPS - 1) {                     // the segment is complete
+                    const int seg = wave + (j / SPS) * nwaves;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) gf_part[(seg * 4 + v) * 64 + lane] = acc[v];
+                    acc = (gg_f32x4){0.f, 0.f, 0.f, 0.f};
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // element (v, lane): row m = 4 lg + v, column n0 + li; segments in ascending order
+    for (int e = tid; e < 256; e += blockDim.x) {
+        const int l = e & 63, v = e >> 6;
+        const int m = 4 * (l >> 4) + v, n = n0 + (l & 15);
+        if (m >= M || n >= N) continue;
+        float sum = 0.f;
+        for (int seg = 0; seg < nseg; ++seg) sum += gf_part[(seg * 4 + v) * 64 + l];
+        C[(size_t)m * ldc + n] = tl_from_float<TO>(sum + (bias ? bias[n] : 0.f));
+    }
+}
+
 template <typename TA, typename TW, typename TO>
 static int gg_launch(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, int lda, int ldc,
                      hipStream_t stream) {
@@ -171,7 +278,13 @@ static int gg_launch(const void* A, const void* W, const float* bias, void* C, i
         hipLaunchKernelGGL((gemm_generic_kernel<TA, TW, TO, WM, WN, MB, NB>), grid, block, 0, stream,            \
                            (const TA*)A, (const TW*)W, bias, (TO*)C, M, N, K, lda, ldc, a_vec, w_vec);           \
     } while (0)
-    if (M <= 32)
+    const int nseg = tl_ceil_div(K, GF_SEG);
+    if (M <= 16 && nseg <= GF_MAX_SEGMENTS) {
+        const int waves = nseg < GF_WAVES ? nseg : GF_WAVES;
+        const size_t lds = (size_t)nseg * 4 * 64 * sizeof(float);
+        hipLaunchKernelGGL((gemm_fewrows_kernel<TA, TW, TO>), dim3(tl_ceil_div(N, 16)), dim3(64 * waves), lds, stream,
+                           (const TA*)A, (const TW*)W, bias, (TO*)C, M, N, K, lda, ldc, a_vec, w_vec);
+    } else if (M <= 32)
         GG_GO(1, 4, 2, 1);        // 32 x 64
     else if (M <= 64)
         GG_GO(1, 4, 4, 2);        // 64 x 128

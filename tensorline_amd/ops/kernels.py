@@ -311,6 +311,7 @@ def linear(a: torch.Tensor | NormedRows, weight: torch.Tensor, bias: torch.Tenso
 
 
 MAX_KEY_SPLITS = 1024    # key splits the attention merge kernel takes
+GENERIC_SPLIT_KEYS = 256  # keys per split of the any-shape attention kernel in steps of one token per sequence
 SKINNY_MAX_ROWS = 16     # rows the few-row kernel serves (one 16-row MFMA tile)
 ROWS64_MAX_ROWS = 64     # rows the 17..64-row kernel serves; above that the library
 
@@ -698,9 +699,19 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         q_start[1:] = torch.cumsum(counts, 0)
         max_query_len = int(counts.max().item()) if T else 1
     _check(head_dim % 16 == 0 and head_dim <= 256, f"paged_attention: head size {head_dim} must be a multiple of 16, at most 256")
+    # Steps of one token per sequence split the keys into runs of GENERIC_SPLIT_KEYS at absolute positions
+    # (longer runs only where the longest context the engine ever runs would need more splits than a launch
+    # takes), whatever the batch: one work-group per sequence and key/value head would walk a long context alone.
+    split_len, nsplit, ws = 0, 1, None
+    if plan is not None and plan.decode_only and max_query_len == 1 and split_keys != 0:
+        split_len, nsplit = _fit_key_splits(int(split_keys) if split_keys else GENERIC_SPLIT_KEYS, plan.max_context,
+                                            plan.fit_context)
+        _check(split_len % 64 == 0, "paged_attention: a split of the any-shape kernel is a multiple of 64 keys")
+        if nsplit > 1:
+            ws = torch.empty(T * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
     _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
           _ptr(q_start), _ptr(pos), _ptr(out), o_stride, _code(q, "paged_attention"), T, S, max(max_query_len, 1), num_heads,
-          num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), _stream())
+          num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nsplit, split_len, _ptr(ws), _stream())
     return out
 
 

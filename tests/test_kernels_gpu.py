@@ -116,6 +116,25 @@ def test_linear_many_rows_keeps_its_shares_on_request():
     assert isinstance(small, torch.Tensor)
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("N,Kd", [(1000, 1184), (3584, 18944), (50, 1030), (70, 513), (130, 7), (16, 512), (37, 40000)])
+def test_linear_few_rows_float32(M, N, Kd):
+    """The float product for at most 16 rows: K in segments of 512 shared by a work-group's waves (one
+    segment, a partial last one, more segments than waves, a K that is no multiple of 4 and one too
+    long for the segments' sums in LDS, which the many-row kernel takes), N no multiple of 16.  A
+    row's result has the same bits whatever other rows come along."""
+    torch.manual_seed(M + N)
+    a = torch.randn(M, Kd, device=DEV)
+    w = torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)
+    b = torch.randn(N, device=DEV)
+    want = a.double() @ w.double().T + b.double()
+    got = K().linear(a, w, b)
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got.double(), want, atol=1e-5, rtol=1e-5)
+    alone = K().linear(a[M - 1:].contiguous(), w, b)
+    torch.testing.assert_close(alone[0], got[M - 1], atol=0, rtol=0)
+
+
 @pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 48, 64])
 @pytest.mark.parametrize("N,Kd", [(1000, 1184), (4608, 3584), (136, 8), (50, 264), (3584, 18944)])
 def test_linear_few_rows_bfloat16(M, N, Kd):
@@ -419,6 +438,18 @@ def test_attention_decode_long_contexts(lens, split):
     splits the merge takes the splits grow; a far key dominates."""
     got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, lens, None, spike=True, seed=5, path="mfma", split_keys=split)
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("lens,split,d,bs", [([33000], None, 128, 16), ([5000, 9, 257], None, 48, 8), ([5000, 256], 512, 64, 24),
+                                              ([1300, 70], 0, 128, 16)])
+def test_attention_any_shape_kernel_splits_keys_in_one_token_steps(dtype, lens, split, d, bs):
+    """The any-shape kernel (the float32 path's attention) in steps of one token per sequence: keys in
+    runs of 256 (or as asked) at absolute positions, a work-group per run, merged by a second kernel;
+    a far key dominates, contexts of a few keys beside thousands, a context that ends exactly at a
+    run's edge, pages of no power of two.  0: no split, the same kernel walking all keys."""
+    got, want = _attention_case(dtype, 6, 2, d, bs, lens, None, spike=True, seed=11, path="generic", split_keys=split)
+    torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
 
 
 @pytest.mark.parametrize("d,bs", [(128, 8), (128, 16), (128, 32), (128, 64), (128, 128), (128, 24), (64, 8), (64, 16),
