@@ -33,6 +33,7 @@
 #define AG_WROWS 16   // rows per wave
 
 #define AG_MAXC 8     // 16-byte pieces of a tile's keys (and of its values) a thread moves
+#define AG_KT(D) ((D) <= 128 ? 64 : 32)   // keys per tile for head size D
 
 template <typename T>
 __device__ __forceinline__ float ag_load(const T* p) { return tl_to_float(*p); }
@@ -79,12 +80,17 @@ template <typename T, int DB>    // DB: blocks of 16 head dimensions (d / 16), 1
 __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
-    T* __restrict__ out, int out_stride, int tiles_per_seq, int QT, int GC, int nq, int nkv, int bs, int KT,
+    T* __restrict__ out, int out_stride, int tiles_per_seq, int QT, int GC, int nq, int nkv, int bs, int bs_shift,
     int window, float scale, int nsplit, int split_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
     constexpr int d = DB * 16;
+    constexpr int KT = AG_KT(d);
     extern __shared__ float smem[];
     constexpr int ks_ld = d + 4;
-    const int vt_ld = KT + 4, ps_ld = KT + 4;
+    constexpr int vt_ld = KT + 4, ps_ld = KT + 4;
+    // the page that holds a key and the key's place in it: a shift and a mask for pages of a power of two
+    // of tokens (bs_shift >= 0), which spares the loader two divisions per piece
+    auto page_of = [&](int key) { return bs_shift >= 0 ? key >> bs_shift : key / bs; };
+    auto in_page = [&](int key) { return bs_shift >= 0 ? key & (bs - 1) : key % bs; };
     float* Ks = smem;
     float* Vt = Ks + KT * ks_ld;
     float* Ps = Vt + d * vt_ld;
@@ -166,8 +172,8 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     // otherwise values are fetched one by one).
     constexpr int E = AgPiece<T>::E;
     constexpr int cpr = d / E;                             // pieces per key
-    const int vpc = KT / E;                                // pieces per head dimension
-    const int pieces = KT * cpr;                           // == d * vpc, at most AG_MAXC * AG_THREADS
+    constexpr int vpc = KT / E;                            // pieces per head dimension
+    constexpr int pieces = KT * cpr;                       // == d * vpc, at most AG_MAXC * AG_THREADS
     const bool v_pieces = (bs % E) == 0;
     uint4 kreg[AG_MAXC], vreg[AG_MAXC];
 
@@ -182,11 +188,11 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
             qi = (qi < pieces) ? qi : pieces - 1;
             int key = k0 + qi / cpr;
             key = (key < k_hi) ? key : k_hi - 1;
-            krow[it] = table[key / bs] * bs + key % bs;
+            krow[it] = table[page_of(key)] * bs + in_page(key);
             const int c = qi / vpc;
             int vkey = k0 + (qi - c * vpc) * E;
             vkey = (vkey < k_hi) ? vkey : ((k_hi - 1) / E) * E;
-            vpage[it] = table[vkey / bs];
+            vpage[it] = table[page_of(vkey)];
         }
 #pragma unroll
         for (int it = 0; it < AG_MAXC; ++it) {
@@ -198,7 +204,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
                 const int c = qi / vpc;
                 int vkey = k0 + (qi - c * vpc) * E;
                 vkey = (vkey < k_hi) ? vkey : ((k_hi - 1) / E) * E;
-                vreg[it] = *reinterpret_cast<const uint4*>(v_cache + (((size_t)vpage[it] * nkv + kvh) * d + c) * bs + vkey % bs);
+                vreg[it] = *reinterpret_cast<const uint4*>(v_cache + (((size_t)vpage[it] * nkv + kvh) * d + c) * bs + in_page(vkey));
             }
         }
     };
@@ -231,8 +237,8 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
                 const int key = k0 + j;
                 float v = 0.f;
                 if (key < k_hi) {
-                    const int page = table[key / bs];
-                    v = ag_load(v_cache + (((size_t)page * nkv + kvh) * d + c) * bs + key % bs);
+                    const int page = table[page_of(key)];
+                    v = ag_load(v_cache + (((size_t)page * nkv + kvh) * d + c) * bs + in_page(key));
                 }
                 Vt[c * vt_ld + j] = v;
             }
@@ -247,7 +253,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
         k_first = (k_first > sp * split_keys) ? k_first : sp * split_keys;
         k_end = (k_end < (sp + 1) * split_keys) ? k_end : (sp + 1) * split_keys;
     }
-    const int key_blocks = KT / 16;
+    constexpr int key_blocks = KT / 16;
     if (k_first < k_end) fetch(k_first);
     for (int k0 = k_first; k0 < k_end; k0 += KT) {
         to_lds(k0);
@@ -420,15 +426,18 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
     const int tiles_per_seq = tl_ceil_div(max_query_len, QT);
     const long long groups = (long long)S * tiles_per_seq;
     TL_CHECK_ARG(groups <= 0x7fffffffLL, "tl_attention_generic: too many work-groups");
-    const int KT = (d <= 128) ? 64 : 32;
+    const int KT = AG_KT(d);
     const size_t smem = ag_lds_bytes(d, KT);
+    int bs_shift = -1;
+    if ((bs & (bs - 1)) == 0)
+        for (bs_shift = 0; (1 << bs_shift) < bs;) ++bs_shift;
     TL_CHECK_ARG(smem <= 160 * 1024, "tl_attention_generic: head size %d needs %zu bytes of LDS", d, smem);
     TL_CHECK_ARG(KT * d / 4 <= AG_MAXC * AG_THREADS, "tl_attention_generic: a tile of head size %d has too many pieces", d);
     dim3 grid((unsigned)groups, nkv, chunks * nsplit), block(AG_THREADS);
 #define AG_LAUNCH(TT, DB)                                                                                             \
     hipLaunchKernelGGL((attn_generic_kernel<TT, DB>), grid, block, smem, stream, (const TT*)q, q_stride,              \
                        (const TT*)k_cache, (const TT*)v_cache, tables, NB, q_start, pos, (TT*)out, out_stride,          \
-                       tiles_per_seq, QT, GC, nq, nkv, bs, KT, window, scale, nsplit, split_keys, ws_o, ws_ml)
+                       tiles_per_seq, QT, GC, nq, nkv, bs, bs_shift, window, scale, nsplit, split_keys, ws_o, ws_ml)
 #define AG_CASE(TT, DB) \
     case DB: AG_LAUNCH(TT, DB); break;
 #define AG_DISPATCH(TT)                                                                              \
