@@ -136,10 +136,10 @@ def test_linear_few_rows_float32(M, N, Kd):
 
 
 @pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 48, 64])
-@pytest.mark.parametrize("N,Kd", [(1000, 1184), (4608, 3584), (136, 8), (50, 264), (3584, 18944)])
+@pytest.mark.parametrize("N,Kd", [(1000, 1184), (4608, 3584), (136, 8), (50, 264), (3584, 18944), (5120, 1184), (2090, 72)])
 def test_linear_few_rows_bfloat16(M, N, Kd):
     """The streaming MFMA kernels (up to 16 rows, and 17 to 64): N no multiple of 16 or 128, K with a
-    partial chunk, K cut into shares."""
+    partial chunk, K cut into shares; numbers of tiles that fill the CUs unevenly (224, 288, 320, 131)."""
     torch.manual_seed(M + N)
     a = torch.randn(M, Kd, device=DEV).to(torch.bfloat16)
     w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(torch.bfloat16)
@@ -336,7 +336,7 @@ def test_fused_projection_applies_an_owed_norm(M, Kd):
 
 
 @pytest.mark.parametrize("M", [1, 6, 16, 17, 33, 64])
-@pytest.mark.parametrize("N,Kd", [(176, 64), (1000, 1184), (3584, 18944), (40, 264), (5000, 256)])
+@pytest.mark.parametrize("N,Kd", [(176, 64), (1000, 1184), (3584, 18944), (40, 264), (5000, 256), (5120, 520)])
 def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
     torch.manual_seed(M + N)
     eps = 1e-6
