@@ -1,0 +1,62 @@
+"""Seeded random configurations of the architecture, each with its own random weights, requests
+and way of cutting them into steps, against the plain implementation, in 32-bit and in bfloat16.
+The two fixed configurations of the other tests pin known traps; these walk the sizes between
+them: head sizes in steps of 16 (most of which only the any-shape kernels take), groups of 1 to 7
+query heads, widths and vocabularies that are no power of two, tied and untied heads, pages of 8
+to 64 tokens, and contexts long enough that one-token steps split their keys."""
+import os
+import random
+import tempfile
+
+import numpy as np
+import pytest
+
+from tests import helpers, plain
+
+pytestmark = pytest.mark.gpu
+LIMIT = {"float32": 1e-5, "bfloat16": 2e-2}
+CUTS = {"whole": helpers.steps_whole, "decode": helpers.steps_prefill_then_decode, "portions": helpers.steps_portions,
+        "mixed": helpers.steps_mixed}
+
+
+def _case(seed: int):
+    rng = random.Random(9000 + seed)
+    d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+    nkv = rng.choice([1, 2, 3, 4])
+    nq = nkv * rng.choice([1, 2, 3, 5, 7])
+    cfg = dict(architectures=["Qwen2ForCausalLM"], vocab_size=rng.choice([97, 300, 512, 777, 1000, 2051]),
+               hidden_size=rng.choice([40, 64, 72, 120, 136, 192, 200, 256]),
+               intermediate_size=rng.choice([48, 88, 176, 200, 368, 520]), num_hidden_layers=rng.choice([1, 2, 3]),
+               num_attention_heads=nq, num_key_value_heads=nkv, head_dim=d, rope_theta=rng.choice([1e4, 5e4, 1e6]),
+               rms_norm_eps=rng.choice([1e-6, 1e-5, 3e-6]), tie_word_embeddings=rng.random() < 0.4,
+               max_position_embeddings=1024)
+    page = rng.choice([8, 16, 32, 64])
+    lengths = [rng.choice([1, 2, 7, 31, 33, 64, 65, 100, 130, 257, 300, 530]) for _ in range(rng.choice([2, 3, 4, 5]))]
+    cut = rng.choice(sorted(CUTS))
+    return cfg, page, lengths, cut, rng
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_configuration_matches_plain(seed):
+    from tensorline_amd.config import Qwen2Config
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.replay import TraceSession
+    from tensorline_amd.weights import write_random_model
+    cfg_dict, page, lengths, cut, rng = _case(seed)
+    what = f"seed {seed}: {cfg_dict} page={page} lengths={lengths} cut={cut}"
+    with tempfile.TemporaryDirectory() as tmp:
+        folder = write_random_model(Qwen2Config.from_dict(cfg_dict), os.path.join(tmp, "m"), seed=seed)
+        w, cfg = plain.load_folder(folder)
+        reqs = {f"r{i}": [rng.randrange(cfg_dict["vocab_size"]) for _ in range(n)] for i, n in enumerate(lengths)}
+        want = helpers.plain_logits(w, cfg, reqs)
+        steps = CUTS[cut](reqs)
+        for dtype in ("float32", "bfloat16"):
+            model, _ = load_model(folder, dtype, "cuda:0")
+            session = TraceSession(model, helpers.max_live_tokens(steps, round_to=max(64, page)), page_size=page)
+            got = helpers.collect_logits(session.step, steps)
+            for rid, toks in reqs.items():
+                scale = max(float(np.abs(want[(rid, i)]).max()) for i in range(len(toks)))
+                for i in range(len(toks)):
+                    err = float(np.abs(got[(rid, i)] - want[(rid, i)]).max()) / scale
+                    assert np.isfinite(err) and err < LIMIT[dtype], (what, dtype, rid, i, err)
+            assert session.cache.all_free(), what
