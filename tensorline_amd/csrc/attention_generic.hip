@@ -76,7 +76,12 @@ __device__ __forceinline__ float ag_row16_sum(float v) {
 }
 
 // LDS: Ks [KT][d + 4] | Vt [d][KT + 4] | Ps [4 waves][16][KT + 4] | row_pos [64] | row_lo [64]
-template <typename T, int DB>    // DB: blocks of 16 head dimensions (d / 16), 1..16
+// KW ("keys over waves"): for steps of so few tokens that a work-group's rows fit one wave (at
+// most 16 (token, head) pairs: a decoded token and its group of query heads).  All four waves then
+// take the same 16 rows and one block of 16 keys of each tile each, instead of three of them
+// standing by; a wave keeps its own running maximum, sum and accumulator over its blocks, and the
+// four are put together through LDS at the end, in the order of the waves.
+template <typename T, int DB, bool KW>    // DB: blocks of 16 head dimensions (d / 16), 1..16
 __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos,
@@ -131,7 +136,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
         const int lo = row_lo[r];
         k_lo = (lo < k_lo) ? lo : k_lo;
         k_hi = (p + 1 > k_hi) ? p + 1 : k_hi;
-        if (r / AG_WROWS == wave) {
+        if (r / AG_WROWS == (KW ? 0 : wave)) {
             w_lo = (lo < w_lo) ? lo : w_lo;
             w_hi = (p + 1 > w_hi) ? p + 1 : w_hi;
         }
@@ -140,7 +145,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     // A operand of S = Q K^T: this lane's row is li of the wave's 16; scaled queries, kept in registers
     ag_f32x4 qa[DB];
     {
-        const int row = wave * AG_WROWS + li;
+        const int row = (KW ? 0 : wave * AG_WROWS) + li;
         const int i = row / GC, g = row - i * GC;
         const bool real = row_pos[row] >= 0;
         const T* qrow = q + (size_t)(t_first + (real ? i : 0)) * q_stride + (size_t)(kvh * G + g0 + (real ? g : 0)) * d;
@@ -156,8 +161,8 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     ag_f32x4 acc[DB];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-        my_pos[v] = row_pos[wave * AG_WROWS + 4 * lg + v];
-        my_lo[v] = row_lo[wave * AG_WROWS + 4 * lg + v];
+        my_pos[v] = row_pos[(KW ? 0 : wave * AG_WROWS) + 4 * lg + v];
+        my_lo[v] = row_lo[(KW ? 0 : wave * AG_WROWS) + 4 * lg + v];
         m[v] = -INFINITY;
         l[v] = 0.f;
     }
@@ -260,14 +265,15 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
         __syncthreads();
         if (k0 + KT < k_end) fetch(k0 + KT);
 
-        if (k0 < w_hi && k0 + KT > w_lo) {                 // a tile none of the wave's rows sees is skipped
+        // a tile none of the wave's rows sees is skipped; KW: a wave without a key block of its own stands by
+        if (k0 < w_hi && k0 + KT > w_lo && (!KW || wave < key_blocks)) {
             // ---- S = Q K^T: per block of 16 keys, 4 DB products; lane holds rows 4 lg + v, key li ----
             ag_f32x4 sblk[4];
 #pragma unroll
-            for (int jb = 0; jb < 4; ++jb) {
+            for (int jb = 0; jb < (KW ? 1 : 4); ++jb) {          // KW: sblk[0] is key block `wave`
                 sblk[jb] = (ag_f32x4){0.f, 0.f, 0.f, 0.f};
-                if (jb < key_blocks) {
-                    const float* kr = Ks + (jb * 16 + li) * ks_ld + 4 * lg;
+                if (KW || jb < key_blocks) {
+                    const float* kr = Ks + ((KW ? wave : jb) * 16 + li) * ks_ld + 4 * lg;
 #pragma unroll
                     for (int kk = 0; kk < DB; ++kk) {
                         const float4 kb = *reinterpret_cast<const float4*>(kr + 16 * kk);
@@ -284,8 +290,12 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
                 float sv[4], mx = -INFINITY;
 #pragma unroll
                 for (int jb = 0; jb < 4; ++jb) {
-                    const int key = k0 + jb * 16 + li;
-                    const bool seen = jb < key_blocks && my_pos[v] >= 0 && key <= my_pos[v] && key >= my_lo[v];
+                    if (KW && jb > 0) {
+                        sv[jb] = -INFINITY;
+                        continue;
+                    }
+                    const int key = k0 + (KW ? wave : jb) * 16 + li;
+                    const bool seen = (KW || jb < key_blocks) && my_pos[v] >= 0 && key <= my_pos[v] && key >= my_lo[v];
                     sv[jb] = seen ? sblk[jb][v] : -INFINITY;
                     mx = fmaxf(mx, sv[jb]);
                 }
@@ -307,8 +317,8 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
 #pragma unroll
                 for (int db = 0; db < DB; ++db) acc[db][v] *= alpha;
 #pragma unroll
-                for (int jb = 0; jb < 4; ++jb)
-                    if (jb < key_blocks) Pw[(4 * lg + v) * ps_ld + jb * 16 + li] = sv[jb];
+                for (int jb = 0; jb < (KW ? 1 : 4); ++jb)
+                    if (KW || jb < key_blocks) Pw[(4 * lg + v) * ps_ld + (KW ? wave : jb) * 16 + li] = sv[jb];
             }
             // Pw is written and read by this wave only; LDS operations of a wave complete in order
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -316,8 +326,9 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             // ---- O += P V: A = P (row li, keys 16 kk + 4 lg + v), B = values (keys likewise, dimension li) ----
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                if (kk < key_blocks) {
+            for (int kq = 0; kq < (KW ? 1 : 4); ++kq) {
+                const int kk = KW ? wave : kq;
+                if (KW || kk < key_blocks) {
                     const float4 pa = *reinterpret_cast<const float4*>(Pw + li * ps_ld + 16 * kk + 4 * lg);
 #pragma unroll
                     for (int db = 0; db < DB; ++db) {
@@ -333,6 +344,47 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
         __syncthreads();                                   // the tile is used up: the next one may be loaded
     }
 
+    if (KW) {
+        // The waves' results for the same 16 rows -> LDS (the tiles are used up), then wave 0 adds them in
+        // the order of the waves: M = max m_w, l = sum l_w e^(m_w - M), acc = sum acc_w e^(m_w - M).
+        float* cacc = smem;                                  // [wave][row][d]: 4 * 16 * d floats, within Ks and Vt
+        float* cml = Ps;                                     // [wave][row][2]
+        constexpr int NW = key_blocks < 4 ? key_blocks : 4;  // waves that had a key block
+        if (wave < NW) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int row = 4 * lg + v;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) cacc[(wave * AG_WROWS + row) * d + db * 16 + li] = acc[db][v];
+                if (li == 0) {
+                    cml[(wave * AG_WROWS + row) * 2] = m[v];
+                    cml[(wave * AG_WROWS + row) * 2 + 1] = l[v];
+                }
+            }
+        }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int row = 4 * lg + v;
+            float M = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) M = fmaxf(M, cml[(w * AG_WROWS + row) * 2]);
+            float lsum = 0.f;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) acc[db][v] = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const float mw = cml[(w * AG_WROWS + row) * 2];
+                const float f = (mw > -INFINITY) ? expf(mw - M) : 0.f;   // a wave that saw no key of the row: nothing
+                lsum += f * cml[(w * AG_WROWS + row) * 2 + 1];
+#pragma unroll
+                for (int db = 0; db < DB; ++db) acc[db][v] += f * cacc[(w * AG_WROWS + row) * d + db * 16 + li];
+            }
+            m[v] = M;
+            l[v] = lsum;
+        }
+    }
     // this lane holds output rows 4 lg + v at head dimensions 16 db + li
     if (nsplit > 1) {
         // the split's sums as they are, with their maximum and denominator (a split that holds no key
@@ -365,29 +417,60 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
 }
 
 // out[t, h, :] = sum_s w_s acc_s / sum_s w_s l_s with w_s = exp(m_s - max m), over the splits in
-// ascending order (a split without keys of the row has l_s = 0 and is left out).  One work-group
-// per (row, head), a thread per head dimension.
+// ascending order (a split without keys of the row has l_s = 0, sums of zero and the weight 0).
+// One work-group per (row, head).  First a thread per split: its maximum and denominator, the
+// largest maximum over the group, its weight; then a thread per head dimension adds the splits'
+// sums, eight loads in flight at a time.  Nothing waits for a load that another load depends on.
+#define AG_MAX_SPLITS 1024
+__device__ __forceinline__ float ag_group_max(float v, float* red) {   // red: one float per wave
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, TL_WAVE));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = red[0];
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) r = fmaxf(r, red[w]);
+    return r;
+}
 template <typename T>
 __global__ __launch_bounds__(256) void attn_generic_merge_kernel(const float* __restrict__ ws_o,
                                                                  const float* __restrict__ ws_ml, T* __restrict__ out,
                                                                  int out_stride, int nq, int d, int nsplit) {
-    const int t = blockIdx.x, h = blockIdx.y, dd = threadIdx.x;
-    if (dd >= d) return;
+    __shared__ float wgt[AG_MAX_SPLITS], wl[AG_MAX_SPLITS], red[4];
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const size_t base = ((size_t)t * nq + h) * nsplit;
-    float M = -INFINITY;
-    for (int s = 0; s < nsplit; ++s)
-        if (ws_ml[(base + s) * 2 + 1] > 0.f) M = fmaxf(M, ws_ml[(base + s) * 2]);
-    float num = 0.f, den = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < nsplit; ++s) {
-        const float ls = ws_ml[(base + s) * 2 + 1];
-        if (ls > 0.f) {
-            const float w = expf(ws_ml[(base + s) * 2] - M);
-            num += w * ws_o[(base + s) * d + dd];
-            den += w * ls;
+    const float2* ml = reinterpret_cast<const float2*>(ws_ml) + base;
+    float2 mine[AG_MAX_SPLITS / 256];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < AG_MAX_SPLITS / 256; ++i) {
+        const int sp = tid + i * 256;
+        mine[i] = sp < nsplit ? ml[sp] : make_float2(-INFINITY, 0.f);
+        if (mine[i].y > 0.f) mx = fmaxf(mx, mine[i].x);
+    }
+    const float M = ag_group_max(mx, red);
+#pragma unroll
+    for (int i = 0; i < AG_MAX_SPLITS / 256; ++i) {
+        const int sp = tid + i * 256;
+        if (sp < nsplit) {
+            const float w = mine[i].y > 0.f ? expf(mine[i].x - M) : 0.f;
+            wgt[sp] = w;
+            wl[sp] = w * mine[i].y;
         }
     }
-    out[(size_t)t * out_stride + (size_t)h * d + dd] = tl_from_float<T>(den > 0.f ? num / den : 0.f);
+    __syncthreads();
+    if (tid >= d) return;
+    float den = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) den += wl[sp];
+    const float* acc = ws_o + base * d + tid;
+    float num = 0.f;
+    for (int s0 = 0; s0 < nsplit; s0 += 8) {
+        float a[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] = acc[(size_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * d];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (s0 + j < nsplit) num += wgt[s0 + j] * a[j];
+    }
+    out[(size_t)t * out_stride + (size_t)h * d + tid] = tl_from_float<T>(den > 0.f ? num / den : 0.f);
 }
 
 static size_t ag_lds_bytes(int d, int KT) {
@@ -417,7 +500,7 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
     const int GC = (G < AG_ROWS) ? G : AG_ROWS;           // query heads per work-group
     const int QT = AG_ROWS / GC;                          // tokens per work-group
     const int chunks = tl_ceil_div(G, GC);
-    TL_CHECK_ARG(nsplit >= 1 && (long long)chunks * nsplit <= 65535,
+    TL_CHECK_ARG(nsplit >= 1 && nsplit <= AG_MAX_SPLITS && (long long)chunks * nsplit <= 65535,
                  "tl_attention_generic: %d chunks of query heads x %d key splits are more than a launch takes", chunks, nsplit);
     TL_CHECK_ARG(nsplit == 1 || (ws && split_keys > 0 && split_keys % 64 == 0),
                  "tl_attention_generic: split keys need a workspace and a split length that is a multiple of 64 (%d)", split_keys);
@@ -433,11 +516,16 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
         for (bs_shift = 0; (1 << bs_shift) < bs;) ++bs_shift;
     TL_CHECK_ARG(smem <= 160 * 1024, "tl_attention_generic: head size %d needs %zu bytes of LDS", d, smem);
     TL_CHECK_ARG(KT * d / 4 <= AG_MAXC * AG_THREADS, "tl_attention_generic: a tile of head size %d has too many pieces", d);
+    // a work-group's rows fit one wave: the waves share the keys of a tile instead (at most one token
+    // per work-group then, so that tokens are not held back by the 16-row limit: QT stays as it is)
+    const bool keys_over_waves = max_query_len * GC <= AG_WROWS && max_query_len <= QT;
     dim3 grid((unsigned)groups, nkv, chunks * nsplit), block(AG_THREADS);
-#define AG_LAUNCH(TT, DB)                                                                                             \
-    hipLaunchKernelGGL((attn_generic_kernel<TT, DB>), grid, block, smem, stream, (const TT*)q, q_stride,              \
+#define AG_LAUNCH_KW(TT, DB, KWV)                                                                                     \
+    hipLaunchKernelGGL((attn_generic_kernel<TT, DB, KWV>), grid, block, smem, stream, (const TT*)q, q_stride,         \
                        (const TT*)k_cache, (const TT*)v_cache, tables, NB, q_start, pos, (TT*)out, out_stride,          \
                        tiles_per_seq, QT, GC, nq, nkv, bs, bs_shift, window, scale, nsplit, split_keys, ws_o, ws_ml)
+#define AG_LAUNCH(TT, DB)                                                                                             \
+    if (keys_over_waves) AG_LAUNCH_KW(TT, DB, true); else AG_LAUNCH_KW(TT, DB, false)
 #define AG_CASE(TT, DB) \
     case DB: AG_LAUNCH(TT, DB); break;
 #define AG_DISPATCH(TT)                                                                              \
@@ -456,6 +544,7 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
 #undef AG_DISPATCH
 #undef AG_CASE
 #undef AG_LAUNCH
+#undef AG_LAUNCH_KW
     TL_CHECK_LAUNCH("tl_attention_generic");
     if (nsplit > 1) {
         dim3 mgrid(T, nq);
