@@ -191,7 +191,11 @@ __global__ __launch_bounds__(GG_THREADS) void gemm_generic_kernel(const TA* __re
 #endif
 #define GF_MAX_SEGMENTS 64    // 64 KB of LDS for the segments' sums: K up to 32,768 (beyond: the kernel above)
 
-template <typename TA, typename TW, typename TO>
+// SHUF: W is the matrix-core ordered copy of a float matrix, [ceil(N/16) tiles][ceil(K/16) steps][64
+// lanes][4 values], lane 16 lg + li holding row li of the tile at k = 16 step + 4 lg .. + 4, zero
+// where it pads: a step's load of a wave is 1 KB of consecutive memory (from the row-major matrix it
+// is 16 pieces of 64 bytes, which streams at about two thirds of the rate), and needs no check.
+template <typename TA, typename TW, typename TO, bool SHUF>
 __global__ __launch_bounds__(512) void gemm_fewrows_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
                                                            const float* __restrict__ bias, TO* __restrict__ C, int M,
                                                            int N, int K, int lda, int ldc, int a_vec, int w_vec) {
@@ -210,8 +214,17 @@ __global__ __launch_bounds__(512) void gemm_fewrows_kernel(const TA* __restrict_
     const TW* wrow_any = W + (size_t)(w_ok ? n0 + li : N - 1) * K;
     const TA* arow_any = A + (size_t)(a_ok ? li : 0) * lda;
     const bool pieces_whole = a_vec != 0 && w_vec != 0;
+    const float4* wtile = reinterpret_cast<const float4*>(W) + (size_t)blockIdx.x * ((K + GG_KS - 1) / GG_KS) * 64 + lane;
     auto load_step = [&](int k0, float4& wv, float4& av) {
-        if (pieces_whole && k0 + GG_KS <= K) {                  // the same for the whole wave
+        if (SHUF) {
+            if (k0 >= K) {                                      // past the last segment's end: the copy ends with K
+                wv = av = make_float4(0.f, 0.f, 0.f, 0.f);
+            } else {
+                wv = wtile[(size_t)(k0 / GG_KS) * 64];
+                if (a_vec != 0 && k0 + GG_KS <= K) av = gg_load4_whole<TA>(arow_any + k0 + 4 * lg);
+                else av = gg_load4<TA>(arow, a_ok, k0 + 4 * lg, K, a_vec != 0);
+            }
+        } else if (pieces_whole && k0 + GG_KS <= K) {           // the same for the whole wave
             wv = gg_load4_whole<TW>(wrow_any + k0 + 4 * lg);
             av = gg_load4_whole<TA>(arow_any + k0 + 4 * lg);
         } else {                                              // past K (the last segment's end): zeros
@@ -282,7 +295,7 @@ static int gg_launch(const void* A, const void* W, const float* bias, void* C, i
     if (M <= 16 && nseg <= GF_MAX_SEGMENTS) {
         const int waves = nseg < GF_WAVES ? nseg : GF_WAVES;
         const size_t lds = (size_t)nseg * 4 * 64 * sizeof(float);
-        hipLaunchKernelGGL((gemm_fewrows_kernel<TA, TW, TO>), dim3(tl_ceil_div(N, 16)), dim3(64 * waves), lds, stream,
+        hipLaunchKernelGGL((gemm_fewrows_kernel<TA, TW, TO, false>), dim3(tl_ceil_div(N, 16)), dim3(64 * waves), lds, stream,
                            (const TA*)A, (const TW*)W, bias, (TO*)C, M, N, K, lda, ldc, a_vec, w_vec);
     } else if (M <= 32)
         GG_GO(1, 4, 2, 1);        // 32 x 64
@@ -291,6 +304,29 @@ static int gg_launch(const void* A, const void* W, const float* bias, void* C, i
     else
         GG_GO(2, 2, 4, 4);        // 128 x 128
 #undef GG_GO
+    return 0;
+}
+
+// Whether the few-row kernel takes a product of this K (the segments' sums must fit its LDS).
+extern "C" int tl_gemm_fewrows_takes(int K) { return K > 0 && tl_ceil_div(K, GF_SEG) <= GF_MAX_SEGMENTS ? 1 : 0; }
+
+// The float product for at most 16 rows from the matrix-core ordered copy of W (see gemm_fewrows_kernel,
+// SHUF): A float [M, K] with row stride lda, Ws float [ceil(N/16), ceil(K/16), 64, 4], C float [M, N].
+// The same sums in the same order as tl_gemm_generic gives for these rows.
+extern "C" int tl_gemm_fewrows_shuffled(const float* A, const float* Ws, const float* bias, float* C, int M, int N, int K,
+                                        int lda, int ldc, hipStream_t stream) {
+    TL_CHECK_ARG(M >= 0 && M <= 16 && N > 0 && K > 0, "tl_gemm_fewrows_shuffled: bad sizes M=%d N=%d K=%d", M, N, K);
+    TL_CHECK_ARG(lda >= K && ldc >= N, "tl_gemm_fewrows_shuffled: row strides lda=%d ldc=%d too small for K=%d N=%d", lda, ldc, K, N);
+    TL_CHECK_ARG(tl_gemm_fewrows_takes(K), "tl_gemm_fewrows_shuffled: K=%d is too long for the segments' sums", K);
+    TL_CHECK_ARG(((uintptr_t)Ws % 16) == 0, "tl_gemm_fewrows_shuffled: the weight copy must be 16-byte aligned");
+    if (M == 0) return 0;
+    const int a_vec = ((uintptr_t)A % 16 == 0 && lda % 4 == 0) ? 1 : 0;
+    const int nseg = tl_ceil_div(K, GF_SEG);
+    const int waves = nseg < GF_WAVES ? nseg : GF_WAVES;
+    const size_t lds = (size_t)nseg * 4 * 64 * sizeof(float);
+    hipLaunchKernelGGL((gemm_fewrows_kernel<float, float, float, true>), dim3(tl_ceil_div(N, 16)), dim3(64 * waves), lds, stream,
+                       A, Ws, bias, C, M, N, K, lda, ldc, a_vec, 1);
+    TL_CHECK_LAUNCH("tl_gemm_fewrows_shuffled");
     return 0;
 }
 

@@ -169,7 +169,28 @@ def shuffle_weight(weight: torch.Tensor) -> torch.Tensor | None:
     return padded.view(Np // 16, 16, Kp // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
 
 
+def shuffle_weight_float(weight: torch.Tensor) -> torch.Tensor | None:
+    """The copy of a float32 [N, K] matrix that the few-row float product streams: [ceil(N/16) tiles,
+    ceil(K/16) steps, 64 lanes, 4 values], lane 16*g + r holding row r of the tile at k = 16*step + 4*g
+    .. +4 (the lane's operands of the four products of a step), zero where it pads: one load of a wave
+    is 1 KB of consecutive memory instead of 16 pieces of 64 bytes.  None for other matrices."""
+    if weight.dtype != torch.float32 or weight.dim() != 2:
+        return None
+    N, K = weight.shape
+    Np, Kp = -(-N // 16) * 16, -(-K // 16) * 16
+    if (Np, Kp) != (N, K):
+        padded = torch.zeros(Np, Kp, dtype=weight.dtype, device=weight.device)
+        padded[:N, :K] = weight
+    else:
+        padded = weight
+    return padded.view(Np // 16, 16, Kp // 16, 4, 4).permute(0, 2, 3, 1, 4).contiguous()
+
+
 def _check_shuffled(shuffled: torch.Tensor, N: int, K: int) -> None:
+    if shuffled.dtype == torch.float32:
+        _check(shuffled.is_contiguous() and tuple(shuffled.shape) == (-(-N // 16), -(-K // 16), 4, 16, 4),
+               f"linear: the shuffled float weight copy does not belong to a [{N}, {K}] matrix")
+        return
     _check(shuffled.dtype == torch.bfloat16 and shuffled.is_contiguous()
            and tuple(shuffled.shape) == (-(-N // 16), -(-K // 32), 4, 16, 8),
            f"linear: the shuffled weight copy does not belong to a [{N}, {K}] matrix")
@@ -345,6 +366,10 @@ def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled=None) -> 
         return out
     if _rows64_ok(a, shuffled, M, K, lda):
         return _rows64(a, shuffled, bias, out, M, N, K, lda, ldc, swiglu=False)
+    if (shuffled is not None and shuffled.dtype == torch.float32 and a.dtype == torch.float32 and out.dtype == torch.float32
+            and M <= SKINNY_MAX_ROWS and library().tl_gemm_fewrows_takes(K)):
+        _call("tl_gemm_fewrows_shuffled", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), M, N, K, lda, ldc, _stream())
+        return out
     _call("tl_gemm_generic", _ptr(a), _code(a, "linear input"), _ptr(weight), _code(weight, "linear weight"),
           _ptr(bias), _ptr(out), _code(out, "linear output"), M, N, K, lda, ldc, _stream())
     return out

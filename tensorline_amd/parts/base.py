@@ -63,6 +63,7 @@ class Linear:
         self.weight: torch.Tensor | None = None
         self.bias: torch.Tensor | None = None
         self.shuffled: torch.Tensor | None = None     # the copy few-row bfloat16 products stream
+        self.shuffled_float: torch.Tensor | None = None   # the same for a float32 weight (the 32-bit path's decode steps)
 
     def tensors(self) -> dict[str, TensorDecl]:
         out = {self.name + ".weight": TensorDecl((self.out_features, self.in_features), "normal", self.std, "compute")}
@@ -79,15 +80,21 @@ class Linear:
         that copy, many-row steps hand the row-major one to the library: twice the bytes, for
         which 288 GB of HBM has room."""
         self.shuffled = kernels.shuffle_weight(self.weight)
+        self.shuffled_float = kernels.shuffle_weight_float(self.weight)
         return self
 
     def tensors_kept(self) -> list[torch.Tensor]:
-        return [t for t in (self.weight, self.bias, self.shuffled) if t is not None]
+        return [t for t in (self.weight, self.bias, self.shuffled, self.shuffled_float) if t is not None]
+
+    @property
+    def streamed(self) -> torch.Tensor | None:
+        """The matrix-core ordered copy few-row products stream, of whichever type the weight has."""
+        return self.shuffled if self.shuffled is not None else self.shuffled_float
 
     def __call__(self, x, out_dtype: torch.dtype | None = None, sink=None, with_bias: bool = True,
                  keep_shares: bool = False):
         return kernels.linear(x, self.weight, self.bias if with_bias else None, out_dtype=out_dtype,
-                              shuffled=self.shuffled, sink=sink, keep_shares=keep_shares)
+                              shuffled=self.streamed, sink=sink, keep_shares=keep_shares)
 
 
 def fuse_linears(name: str, parts: list[Linear]) -> Linear:

@@ -47,5 +47,5 @@ class SwiGLU(Part):
     keeps_share_sums = True
 
     def forward(self, h, ctx, sink=None, keep_shares: bool = False):
-        act = kernels.swiglu_gate_up(h, self.gate_up.weight, self.gate_up.shuffled)
+        act = kernels.swiglu_gate_up(h, self.gate_up.weight, self.gate_up.streamed)
         return self.down(act, out_dtype=torch.float32, sink=sink, keep_shares=keep_shares)

@@ -133,6 +133,12 @@ def test_linear_few_rows_float32(M, N, Kd):
     torch.testing.assert_close(got.double(), want, atol=1e-5, rtol=1e-5)
     alone = K().linear(a[M - 1:].contiguous(), w, b)
     torch.testing.assert_close(alone[0], got[M - 1], atol=0, rtol=0)
+    # from the matrix-core ordered copy of the weight (what the engine's decode steps stream): the same bits
+    ws = K().shuffle_weight_float(w)
+    assert ws.shape == (-(-N // 16), -(-Kd // 16), 4, 16, 4)
+    torch.testing.assert_close(K().linear(a, w, b, shuffled=ws), got, atol=0, rtol=0)
+    strided = torch.randn(M, Kd + 5, device=DEV)[:, 1:Kd + 1]          # rows neither aligned nor contiguous
+    torch.testing.assert_close(K().linear(strided, w, b, shuffled=ws), K().linear(strided, w, b), atol=0, rtol=0)
 
 
 @pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 48, 64])
