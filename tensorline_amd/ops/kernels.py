@@ -304,7 +304,7 @@ def linear(a: torch.Tensor | NormedRows, weight: torch.Tensor, bias: torch.Tenso
         _check(out is None and (_skinny_ok(a, shuffled, M, K, lda) or _rows64_ok(a, shuffled, M, K, lda)),
                "linear: a deferred norm needs a streaming bfloat16 kernel (at most 64 rows, a shuffled weight copy)")
         _check_shuffled(shuffled, N, K)
-        few = M <= SKINNY_MAX_ROWS
+        few = M <= SKINNY_MAX_ROWS and not (_few_rows_go_to_rows64(N, K) and _rows64_ok(a, shuffled, M, K, lda, few_too=True))
         # a sink's partials: per 16-column tile where the first kernel completes the sums, per 256 columns
         # where the mid-row product's second kernel does
         per = 16 if few or library().tl_gemm_rows64_shares(M, N, K) == 1 else 256
@@ -342,9 +342,22 @@ def _skinny_ok(a: torch.Tensor, shuffled: torch.Tensor | None, M: int, K: int, l
             and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0)
 
 
-def _rows64_ok(a: torch.Tensor, shuffled: torch.Tensor | None, M: int, K: int, lda: int) -> bool:
-    return (shuffled is not None and a.dtype == torch.bfloat16 and SKINNY_MAX_ROWS < M <= ROWS64_MAX_ROWS
+def _rows64_ok(a: torch.Tensor, shuffled: torch.Tensor | None, M: int, K: int, lda: int, few_too: bool = False) -> bool:
+    return (shuffled is not None and a.dtype == torch.bfloat16 and (few_too or SKINNY_MAX_ROWS < M) and M <= ROWS64_MAX_ROWS
             and K % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0)
+
+
+def _few_rows_go_to_rows64(N: int, K: int) -> bool:
+    """Whether a plain product of at most 16 rows runs on the 17-to-64-row kernel.  The few-row
+    kernel gives every 16-column tile to one work-group, so 320 tiles (5,120 columns) put two on 64
+    of the 256 CUs and one on the rest, and the product takes as long as two tiles; the other
+    kernel cuts K into shares as well and fills whole rounds of CUs, at the price of a second
+    kernel.  That pays where the last round of tiles is far from full and K is long (measured at 8
+    rows: 5,120 x 13,824: 31.6 against 38.0 us, 5,120 x 27,648: 59.4 against 70.4; not at 5,120 x
+    5,120: 15.8 against 13.9).  The choice depends on the matrix alone, not on the rows."""
+    tiles, steps = -(-N // 16), -(-K // 128)
+    rounds = -(-tiles // 256)
+    return 2 <= rounds <= 3 and tiles < 0.75 * rounds * 256 and rounds * steps >= 150
 
 
 def _rows64(a, shuffled, bias, out, M, N, K, lda, ldc, swiglu: bool, norm=None):
@@ -360,11 +373,11 @@ def _linear_dispatch(a, weight, bias, out, M, N, K, lda, ldc, shuffled=None) -> 
     """bfloat16 with few rows: the streaming MFMA kernel.  float32, and shapes that kernel does not
     take: the plain tiled kernel.  (bfloat16 with many rows went to the library before this, where
     the reference uses one too: tensorline/paged.py:179-188.)"""
-    if _skinny_ok(a, shuffled, M, K, lda):
+    if _skinny_ok(a, shuffled, M, K, lda) and not _few_rows_go_to_rows64(N, K):
         _call("tl_gemm_skinny", _ptr(a), _ptr(shuffled), _ptr(bias), _ptr(out), _code(out, "linear output"),
               M, N, K, lda, ldc, None, _stream())
         return out
-    if _rows64_ok(a, shuffled, M, K, lda):
+    if _rows64_ok(a, shuffled, M, K, lda, few_too=True):
         return _rows64(a, shuffled, bias, out, M, N, K, lda, ldc, swiglu=False)
     if (shuffled is not None and shuffled.dtype == torch.float32 and a.dtype == torch.float32 and out.dtype == torch.float32
             and M <= SKINNY_MAX_ROWS and library().tl_gemm_fewrows_takes(K)):

@@ -142,10 +142,13 @@ def test_linear_few_rows_float32(M, N, Kd):
 
 
 @pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 48, 64])
-@pytest.mark.parametrize("N,Kd", [(1000, 1184), (4608, 3584), (136, 8), (50, 264), (3584, 18944), (5120, 1184), (2090, 72)])
+@pytest.mark.parametrize("N,Kd", [(1000, 1184), (4608, 3584), (136, 8), (50, 264), (3584, 18944), (5120, 1184), (2090, 72),
+                                  (5120, 9728)])
 def test_linear_few_rows_bfloat16(M, N, Kd):
     """The streaming MFMA kernels (up to 16 rows, and 17 to 64): N no multiple of 16 or 128, K with a
-    partial chunk, K cut into shares; numbers of tiles that fill the CUs unevenly (224, 288, 320, 131)."""
+    partial chunk, K cut into shares; numbers of tiles that fill the CUs unevenly (224, 288, 320, 131),
+    the last with a K so long that few rows too go to the kernel that cuts K into shares."""
+    assert K()._few_rows_go_to_rows64(N, Kd) == ((N, Kd) == (5120, 9728))
     torch.manual_seed(M + N)
     a = torch.randn(M, Kd, device=DEV).to(torch.bfloat16)
     w = (torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(torch.bfloat16)
@@ -289,7 +292,8 @@ def _normed_rows(h, gamma, eps, parts):
 
 
 @pytest.mark.parametrize("M", [1, 7, 16, 17, 40, 64])
-@pytest.mark.parametrize("N,Kd,parts", [(176, 64, 4), (1000, 1184, 74), (3584, 3584, 224), (50, 264, 1), (37888, 3584, 14)])
+@pytest.mark.parametrize("N,Kd,parts", [(176, 64, 4), (1000, 1184, 74), (3584, 3584, 224), (50, 264, 1), (37888, 3584, 14),
+                                        (5120, 9728, 38)])
 def test_products_apply_an_owed_norm(M, N, Kd, parts):
     """A product of rows h * g with the division by rms(h) owed equals the product of RMSNorm(h) * g:
     plain, gate/up with SiLU, and q/k/v with rotation and cache write."""
@@ -342,7 +346,7 @@ def test_fused_projection_applies_an_owed_norm(M, Kd):
 
 
 @pytest.mark.parametrize("M", [1, 6, 16, 17, 33, 64])
-@pytest.mark.parametrize("N,Kd", [(176, 64), (1000, 1184), (3584, 18944), (40, 264), (5000, 256), (5120, 520)])
+@pytest.mark.parametrize("N,Kd", [(176, 64), (1000, 1184), (3584, 18944), (40, 264), (5000, 256), (5120, 520), (5120, 9728)])
 def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
     torch.manual_seed(M + N)
     eps = 1e-6
