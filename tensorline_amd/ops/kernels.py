@@ -615,10 +615,21 @@ def _singles_get_own_launch(plan, singles: list[int], num_heads: int, num_kv_hea
     return walk_us > portions_us + 9 + stream_us + 5
 
 
+LONG_SPLIT_KEYS = 1024    # the longest split the context scales a split to (64 pages of 16: a wave keeps their ids in its lanes)
+
+
 def _key_splits(num_seqs: int, num_kv_heads: int, max_context: int, fit_context: int = 0) -> tuple[int, int]:
-    """(keys per split, number of splits) for ``num_seqs`` one-token sequences; (0, 1): no split."""
+    """(keys per split, number of splits) for ``num_seqs`` one-token sequences; (0, 1): no split.
+    The length follows the batch (enough waves for the GPU at a context of 4,096) and doubles with
+    every doubling of the step's longest context beyond 4,096, up to LONG_SPLIT_KEYS: a context of
+    32,768 is then cut into as many runs as one of 4,096, not eight times as many for the merge
+    kernel to read back.  The doublings lie where the graphs' context buckets do, so an eager step
+    and the graph captured for its bucket cut alike."""
     base = (1 << max(num_seqs - 1, 0).bit_length()) * num_kv_heads
     split_len = 64 if base <= 8 else 128 if base <= 32 else 256 if base <= 128 else 512 if base <= 512 else 0
+    reach = 4096
+    while split_len and reach < max_context and split_len < LONG_SPLIT_KEYS:
+        split_len, reach = split_len * 2, reach * 2
     return _fit_key_splits(split_len, max_context, fit_context)
 
 

@@ -85,16 +85,21 @@ def test_in_place_update_is_off_for_windowed_caches():
     assert not runner._advance(cap, [StepEntry("a", [1], 6, [0])])
 
 
-def test_key_splits_are_fitted_to_the_longest_context_the_engine_runs():
-    """A graph is captured for the longest context, an eager step sees the real one: both must cut
-    the keys into the same runs, so the length of a split follows the engine's limit where it is
-    known and only the number of splits follows the step."""
-    from tensorline_amd.ops.kernels import MAX_KEY_SPLITS, _fit_key_splits, _key_splits
+def test_key_splits_follow_the_batch_and_the_context_bucket():
+    """A graph is captured for a context bucket, an eager step sees the real context: both must cut
+    the keys into the same runs.  The length of a split follows the batch and doubles with the
+    context where the buckets do (4,096, 8,192, ...), up to 1,024 keys; beyond that, and for split
+    lengths the caller forces, it is fitted to the engine's longest context so that no launch has
+    more splits than the merge takes."""
+    from tensorline_amd.ops.kernels import LONG_SPLIT_KEYS, MAX_KEY_SPLITS, _fit_key_splits, _key_splits
     assert _key_splits(1, 4, 3000) == (64, 47)
-    assert _key_splits(1, 4, 3000, fit_context=4096) == (64, 47)
-    long = 64 * MAX_KEY_SPLITS * 2                        # twice what 1,024 splits of 64 keys cover
-    graph = _key_splits(1, 4, long, fit_context=long)
-    eager = _key_splits(1, 4, 3000, fit_context=long)
-    assert graph == (128, MAX_KEY_SPLITS) and eager == (128, 24)
-    assert _key_splits(1, 4, 3000) == (64, 47)            # without the hint only the step's own context counts
+    assert _key_splits(1, 4, 4096) == (64, 64) and _key_splits(1, 4, 4097) == (128, 33)
+    assert _key_splits(1, 4, 5000) == _key_splits(1, 4, 5000, fit_context=8192) == (128, 40)
+    assert _key_splits(1, 4, 8192)[0] == _key_splits(1, 4, 4200)[0] == 128        # a live context and its bucket cut alike
+    assert _key_splits(8, 4, 32768) == (1024, 32) and _key_splits(8, 4, 32784)[0] == LONG_SPLIT_KEYS
+    assert _key_splits(64, 4, 32768) == (1024, 32)                                # 512 by the batch, capped
+    assert _key_splits(1, 4, 10 ** 6)[0] == LONG_SPLIT_KEYS
+    long = 64 * MAX_KEY_SPLITS * 2                        # a forced length: twice what 1,024 splits of 64 keys cover
+    assert _fit_key_splits(64, long, long) == (128, MAX_KEY_SPLITS) and _fit_key_splits(64, 3000, long) == (128, 24)
+    assert _fit_key_splits(64, 3000) == (64, 47)          # without the hint only the step's own context counts
     assert _fit_key_splits(0, 10 ** 6, 10 ** 7) == (0, 1)
