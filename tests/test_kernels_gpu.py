@@ -452,12 +452,13 @@ def test_attention_decode_long_contexts(lens, split):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("lens,split,d,bs", [([33000], None, 128, 16), ([5000, 9, 257], None, 48, 8), ([5000, 256], 512, 64, 24),
-                                              ([1300, 70], 0, 128, 16)])
+                                              ([1300, 70], 0, 128, 16), ([700, 9, 257], None, 256, 16), ([1025], None, 144, 24)])
 def test_attention_any_shape_kernel_splits_keys_in_one_token_steps(dtype, lens, split, d, bs):
     """The any-shape kernel (the float32 path's attention) in steps of one token per sequence: keys in
     runs of 256 (or as asked) at absolute positions, a work-group per run, merged by a second kernel;
     a far key dominates, contexts of a few keys beside thousands, a context that ends exactly at a
-    run's edge, pages of no power of two.  0: no split, the same kernel walking all keys."""
+    run's edge, pages of no power of two, head sizes above 128 (tiles of 32 keys: two of the four
+    waves have a key block).  0: no split, the same kernel walking all keys."""
     got, want = _attention_case(dtype, 6, 2, d, bs, lens, None, spike=True, seed=11, path="generic", split_keys=split)
     torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
 
