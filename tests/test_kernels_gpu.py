@@ -372,8 +372,9 @@ def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
 
 
 def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False, path=None, split_keys=None,
-                    route_singles=None):
-    """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries."""
+                    route_singles=None, pool_pages=None):
+    """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries.
+    pool_pages: the sequences' pages are the last ones of a pool of that many."""
     torch.manual_seed(seed)
     S = len(lens)
     q_lens = q_lens or [1] * S
@@ -382,6 +383,12 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
     kc = torch.randn(num_blocks, bs, nkv, d, device=DEV).to(dtype)
     vc = torch.randn(num_blocks, nkv, d, bs, device=DEV).to(dtype)
     tables = torch.randperm(num_blocks, device=DEV)[:S * nb].view(S, nb).to(torch.int32)   # scattered pages
+    if pool_pages:
+        first = pool_pages - num_blocks
+        big_k = torch.zeros(pool_pages, bs, nkv, d, dtype=dtype, device=DEV)
+        big_v = torch.zeros(pool_pages, nkv, d, bs, dtype=dtype, device=DEV)
+        big_k[first:], big_v[first:] = kc, vc
+        kc, vc, tables = big_k, big_v, tables + first
     seq_of, pos = [], []
     for s, (n, ql) in enumerate(zip(lens, q_lens)):
         for p in range(n - ql, n):
@@ -412,6 +419,8 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
                               q_start=torch.tensor(qs, dtype=torch.int32, device=DEV),
                               ctx_start=torch.tensor(plan.starts, dtype=torch.int32, device=DEV), plan=plan,
                               path=path, split_keys=split_keys, single_seqs=single_seqs, route_singles=route_singles)
+    if pool_pages:
+        kc, vc, tables = kc[first:], vc[first:], tables - first
     kf, vf = kc.double().cpu().view(-1, nkv, d), vc.double().cpu().permute(0, 3, 1, 2).reshape(-1, nkv, d)
     want = torch.empty(T, nq, d, dtype=torch.float64)
     tcpu = tables.cpu().long()
@@ -440,6 +449,68 @@ def test_attention_portions_and_spike(dtype, nq, nkv, d, bs):
     lens, q_lens = [70, 9, 300, 2], [33, 9, 2, 1]
     got, want = _attention_case(dtype, nq, nkv, d, bs, lens, q_lens, spike=True, seed=3)
     torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
+
+
+def _pages_beyond_32_bits(bs, nkv, d):
+    """Pages of a pool whose planes hold more than 2^31 elements (2^32 bytes and more)."""
+    return (1 << 31) // (bs * nkv * d) + 4096
+
+
+@pytest.mark.parametrize("dtype,path", [(torch.bfloat16, "mfma"), (torch.bfloat16, "generic"), (torch.float32, "generic")])
+def test_attention_reads_pages_at_offsets_beyond_32_bits(dtype, path):
+    """The sequences' pages are the last ones of a pool of several GB per plane: a page's offset in
+    elements is above 2^31 and must be computed in 64 bits, in one-token steps and in portions."""
+    nq, nkv, d, bs = 4, 2, 128, 16
+    pool = _pages_beyond_32_bits(bs, nkv, d)
+    try:
+        for lens, q_lens in (([700, 33], None), ([300, 40, 65], [33, 40, 1])):
+            got, want = _attention_case(dtype, nq, nkv, d, bs, lens, q_lens, spike=True, seed=11, path=path, pool_pages=pool)
+            torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
+    finally:
+        torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_cache_writes_at_offsets_beyond_32_bits(dtype):
+    """The kernels that write the cache (rotation and store; the fused projections for few rows and
+    for 17 to 64 rows) with slots on the last pages of a pool of several GB per plane leave there
+    what they leave in a small pool, and nothing anywhere else."""
+    nq, nkv, d, bs, Kd, small = 4, 2, 128, 16, 3584, 12
+    pool = _pages_beyond_32_bits(bs, nkv, d)
+    first = pool - small
+    torch.manual_seed(4)
+    inv_freq = (1e6 ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)).float().to(DEV)
+    N = (nq + 2 * nkv) * d
+    try:
+        big_k = torch.zeros(pool, bs, nkv, d, dtype=dtype, device=DEV)
+        big_v = torch.zeros(pool, nkv, d, bs, dtype=dtype, device=DEV)
+        for M in (5, 40):
+            pos = torch.randint(0, 4000, (M,), dtype=torch.int32, device=DEV)
+            slots = torch.randperm(small * bs, device=DEV)[:M].to(torch.int32)
+            writers = [lambda kc, vc, sl: K().rope_store(qkv.clone(), pos, inv_freq, nq, nkv, d, kc, vc, sl)]
+            qkv = torch.randn(M, N, device=DEV).to(dtype)
+            if dtype == torch.bfloat16:
+                h = torch.randn(M, Kd, device=DEV).to(dtype)
+                ws = K().shuffle_weight((torch.randn(N, Kd, device=DEV) / math.sqrt(Kd)).to(dtype))
+                b = torch.randn(N, device=DEV)
+                fused = lambda kc, vc, sl: K().qkv_rope_store(h, ws, b, pos, inv_freq, nq, nkv, d, kc, vc, sl)
+                assert fused(torch.zeros(small, bs, nkv, d, dtype=dtype, device=DEV),
+                             torch.zeros(small, nkv, d, bs, dtype=dtype, device=DEV), slots) is not None
+                writers.append(fused)
+            for write in writers:
+                kc = torch.zeros(small, bs, nkv, d, dtype=dtype, device=DEV)
+                vc = torch.zeros(small, nkv, d, bs, dtype=dtype, device=DEV)
+                write(kc, vc, slots)
+                assert kc.abs().sum() > 0 and vc.abs().sum() > 0
+                big_k[first:].zero_()
+                big_v[first:].zero_()
+                write(big_k, big_v, slots + first * bs)
+                assert torch.equal(big_k[first:], kc) and torch.equal(big_v[first:], vc)
+        # nothing was written below the last pages (a 32-bit offset would land there)
+        assert not big_k[:first].any() and not big_v[:first].any()
+    finally:
+        del big_k, big_v
+        torch.cuda.empty_cache()
 
 
 @pytest.mark.parametrize("lens,split", [([33000], None), ([70001, 9], None), ([70001], 32)])
