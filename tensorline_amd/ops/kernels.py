@@ -645,6 +645,12 @@ def _fit_key_splits(split_len: int, max_context: int, fit_context: int = 0) -> t
     return split_len, max(1, -(-max_context // split_len))
 
 
+def attention_takes_head_dim(head_dim: int) -> bool:
+    """The head sizes the attention kernels take: multiples of 16 up to 256 (32, 64 and 128 on the
+    bfloat16 MFMA kernels, the others on the any-shape kernel)."""
+    return head_dim > 0 and head_dim % 16 == 0 and head_dim <= 256
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, tables: torch.Tensor,
                     seq_of_token: torch.Tensor, pos: torch.Tensor, num_heads: int, num_kv_heads: int,
                     head_dim: int, scale: float, window: int = 0, out: torch.Tensor | None = None,
@@ -747,7 +753,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         q_start = torch.zeros(S + 1, dtype=torch.int32, device=q.device)
         q_start[1:] = torch.cumsum(counts, 0)
         max_query_len = int(counts.max().item()) if T else 1
-    _check(head_dim % 16 == 0 and head_dim <= 256, f"paged_attention: head size {head_dim} must be a multiple of 16, at most 256")
+    _check(attention_takes_head_dim(head_dim), f"paged_attention: head size {head_dim} must be a multiple of 16, at most 256")
     # Steps of one token per sequence split the keys into runs of GENERIC_SPLIT_KEYS at absolute positions
     # (longer runs only where the longest context the engine ever runs would need more splits than a launch
     # takes), whatever the batch: one work-group per sequence and key/value head would walk a long context alone.

@@ -30,6 +30,9 @@ class PagedAttention(Part):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
         self.num_heads, self.num_kv_heads, self.head_dim = int(num_heads), int(num_kv_heads), int(head_dim)
+        if not kernels.attention_takes_head_dim(self.head_dim):
+            raise ValueError(f"{prefix}: a head size of {self.head_dim} is not served: the attention kernels take "
+                             "multiples of 16 up to 256")
         self.window = int(window or 0)
         self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
         self.kv_proj = bool(kv_proj)

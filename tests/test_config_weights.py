@@ -56,6 +56,18 @@ def test_registry(tmp_path):
     assert len(spec.layers) == 2 and spec.layers[1].mixer.params["num_heads"] == 6
 
 
+@pytest.mark.parametrize("head_dim", [8, 40, 272])
+def test_head_sizes_no_kernel_serves_are_refused_when_the_model_is_built(head_dim):
+    """The configuration allows any even head size; the attention part refuses, before any weight is
+    read, those the kernels do not take, instead of failing in the first step."""
+    from tensorline_amd.models.decoder import DecoderModel
+    arch = get_architecture("Qwen2ForCausalLM")
+    spec = arch.build_spec(Qwen2Config.from_dict(dict(BASE, head_dim=head_dim)))
+    with pytest.raises(ValueError, match=f"head size of {head_dim}"):
+        DecoderModel(spec, torch.float32, "cpu")
+    DecoderModel(arch.build_spec(Qwen2Config.from_dict(dict(BASE, head_dim=48))), torch.float32, "cpu")
+
+
 def test_engine_config_names():
     e = EngineConfig(dtype="bf16")
     assert (e.dtype, e.block_size, e.max_num_seqs, e.max_batched_tokens, e.max_model_len) == ("bfloat16", 16, 64, 2048, 4096)

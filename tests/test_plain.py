@@ -130,7 +130,7 @@ def _tiny(tied):
     from tensorline_amd.models.qwen2 import qwen2_spec
     from tensorline_amd.weights.random_init import random_tensor
     cfg = dict(vocab_size=50, hidden_size=24, intermediate_size=40, num_hidden_layers=2, num_attention_heads=3,
-               num_key_value_heads=1, head_dim=8, rope_theta=100.0, rms_norm_eps=1e-5, tie_word_embeddings=tied)
+               num_key_value_heads=1, head_dim=16, rope_theta=100.0, rms_norm_eps=1e-5, tie_word_embeddings=tied)
     model = DecoderModel(qwen2_spec(Qwen2Config.from_dict(dict(cfg, architectures=["Qwen2ForCausalLM"]))), torch.float32, "cpu")
     w = {n: random_tensor(n, d, 1).double() for n, d in model.tensor_decls().items()}
     return w, cfg
@@ -155,7 +155,7 @@ def test_model_layer_composition_by_hand():
     x = w["model.embed_tokens.weight"][ids]
     p = "model.layers.0."
     a = plain.attention_block(plain.rmsnorm(x, w[p + "input_layernorm.weight"], 1e-5), w, p + "self_attn.",
-                              torch.arange(3), 3, 1, 8, 100.0)
+                              torch.arange(3), 3, 1, 16, 100.0)
     x = x + a
     x = x + plain.swiglu(plain.rmsnorm(x, w[p + "post_attention_layernorm.weight"], 1e-5), w[p + "mlp.gate_proj.weight"],
                          w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
@@ -167,8 +167,8 @@ def test_attention_block_depends_on_distances_only():
     w, cfg = _tiny(tied=False)
     h = torch.randn(5, 24, dtype=torch.float64)
     p = "model.layers.0.self_attn."
-    a = plain.attention_block(h, w, p, torch.arange(5), 3, 1, 8, 100.0)
-    b = plain.attention_block(h, w, p, torch.arange(5) + 300, 3, 1, 8, 100.0)
+    a = plain.attention_block(h, w, p, torch.arange(5), 3, 1, 16, 100.0)
+    b = plain.attention_block(h, w, p, torch.arange(5) + 300, 3, 1, 16, 100.0)
     torch.testing.assert_close(a, b, atol=1e-5, rtol=1e-5)         # float32 angles at position ~300 cost a little
 
 

@@ -36,14 +36,11 @@ def _case(seed: int):
     return cfg, page, lengths, cut, rng
 
 
-@pytest.mark.parametrize("seed", range(24))
-def test_random_configuration_matches_plain(seed):
+def _compare(cfg_dict, page, lengths, cut, rng, seed, what):
     from tensorline_amd.config import Qwen2Config
     from tensorline_amd.engine.loading import load_model
     from tensorline_amd.engine.replay import TraceSession
     from tensorline_amd.weights import write_random_model
-    cfg_dict, page, lengths, cut, rng = _case(seed)
-    what = f"seed {seed}: {cfg_dict} page={page} lengths={lengths} cut={cut}"
     with tempfile.TemporaryDirectory() as tmp:
         folder = write_random_model(Qwen2Config.from_dict(cfg_dict), os.path.join(tmp, "m"), seed=seed)
         w, cfg = plain.load_folder(folder)
@@ -60,3 +57,24 @@ def test_random_configuration_matches_plain(seed):
                     err = float(np.abs(got[(rid, i)] - want[(rid, i)]).max()) / scale
                     assert np.isfinite(err) and err < LIMIT[dtype], (what, dtype, rid, i, err)
             assert session.cache.all_free(), what
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_configuration_matches_plain(seed):
+    cfg_dict, page, lengths, cut, rng = _case(seed)
+    _compare(cfg_dict, page, lengths, cut, rng, seed, f"seed {seed}: {cfg_dict} page={page} lengths={lengths} cut={cut}")
+
+
+@pytest.mark.parametrize("hidden,inter,vocab,d", [(50, 90, 97, 16), (7, 9, 11, 16), (100, 25, 33, 48), (1, 1, 2, 16),
+                                                  (136, 88, 300, 160), (72, 176, 777, 256)])
+@pytest.mark.parametrize("cut", sorted(CUTS))
+def test_odd_widths_and_large_heads_match_plain(hidden, inter, vocab, d, cut):
+    """Widths that are no multiple of 8 (rows of the weights are not 16-byte aligned, so no streaming
+    kernel takes them), down to a width of one, and head sizes above 128 through the whole model."""
+    rng = random.Random(hidden * 1000 + d)
+    nkv = rng.choice([1, 2, 3])
+    cfg_dict = dict(architectures=["Qwen2ForCausalLM"], vocab_size=vocab, hidden_size=hidden, intermediate_size=inter,
+                    num_hidden_layers=2, num_attention_heads=nkv * rng.choice([1, 2, 3]), num_key_value_heads=nkv, head_dim=d,
+                    rope_theta=1e4, rms_norm_eps=1e-6, tie_word_embeddings=hidden % 4 == 0, max_position_embeddings=1024)
+    page, lengths = rng.choice([8, 16, 32]), [rng.choice([2, 33, 65, 130]) for _ in range(3)]
+    _compare(cfg_dict, page, lengths, cut, rng, hidden, f"{cfg_dict} page={page} lengths={lengths} cut={cut}")
