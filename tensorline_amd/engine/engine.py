@@ -66,6 +66,7 @@ class InferenceEngine:
     def add_request(self, prompt_tokens: list[int], params: SamplingParams | None = None,
                     stats: GenStats | None = None) -> Request:
         params = params or SamplingParams()
+        params.validate()
         toks = [int(t) for t in prompt_tokens]
         V = self.model.vocab_size
         if any(t < 0 or t >= V for t in toks):

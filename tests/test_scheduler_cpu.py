@@ -128,6 +128,19 @@ def test_abort_frees_pages(tiny, cpu_kernels):
     eng.abort(a)                                                   # a second abort is a no-op
 
 
+@pytest.mark.parametrize("bad,word", [(dict(max_tokens=0), "max_tokens"), (dict(max_tokens=2.5), "max_tokens"),
+                                      (dict(temperature=float("nan")), "temperature"), (dict(top_p=0.0), "top_p"),
+                                      (dict(top_p=-0.1), "top_p"), (dict(top_p=float("nan")), "top_p")])
+def test_options_without_a_sampling_rule_are_refused_when_added(tiny, cpu_kernels, bad, word):
+    d, prompts, _ = tiny
+    eng = make_engine(d)
+    with pytest.raises(ValueError, match=word):
+        eng.add_request(prompts[1], SamplingParams(**bad))
+    assert not eng.has_work() and eng.cache.all_free()
+    eng.add_request(prompts[1], SamplingParams(max_tokens=1, temperature=-1.0, top_p=1.5))    # greedy; keeps every token
+    eng.run_until_done()
+
+
 def test_temperature_sampling_is_seeded_and_batch_independent(tiny, cpu_kernels):
     d, prompts, _ = tiny
     sp = lambda seed: SamplingParams(12, temperature=0.9, top_p=0.8, stop_token_ids=NO_STOP, seed=seed)
