@@ -19,7 +19,7 @@ class EngineConfig:
     graph_warmup_tokens: int = 512       # capture graphs for contexts up to this many tokens at start-up
     prefix_caching: bool = True
     overlap: bool = True                 # queue decode step t + 1 before reading step t's tokens (--no-overlap there)
-    tune_library: bool = False           # at start-up, let the library pick its kernels for full prompt portions by measurement
+    tune_library: bool = False           # at start-up, let the library pick its kernels by measurement: full prompt portions, decode steps above 64 rows
     device: str = "cuda:0"
 
     def __post_init__(self):

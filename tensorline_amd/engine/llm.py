@@ -67,6 +67,12 @@ class LLM:
             from tensorline_amd.engine.graphs import GraphRunner
             runner = GraphRunner(self.model, self.cache, max_batch=ec.max_num_seqs,
                                  max_blocks_per_seq=-(-ec.max_model_len // ec.block_size))
+            if ec.tune_library and self.model.dtype == torch.bfloat16:
+                # decode steps of more rows than the engine's own kernels take are library products too,
+                # of exactly the graphs' row counts
+                for rows in runner.batch_buckets:
+                    if rows > kernels.ROWS64_MAX_ROWS and rows != ec.max_batched_tokens:
+                        self.model.tune_library(rows)
             if ec.graph_warmup_tokens:
                 runner.warmup(min(ec.graph_warmup_tokens, ec.max_model_len))
         self.engine = InferenceEngine(self.model, self.cache, max_num_seqs=ec.max_num_seqs,

@@ -311,10 +311,10 @@ def test_graph_decode_matches_eager_and_isolates_padding(folder_b):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("rows, bucket", [(19, 32), (41, 64)])
+@pytest.mark.parametrize("rows, bucket", [(19, 32), (41, 64), (70, 128)])
 def test_graph_replay_of_wide_buckets_matches_plain(case, rows, bucket, dtype):
-    """Graphs of 32 and of 64 rows (the 17-to-64-row kernels inside a captured graph), with padding
-    rows: 12 decode steps whose logits are the plain implementation's at every row and step, on
+    """Graphs of 32 and of 64 rows (the 17-to-64-row kernels inside a captured graph) and of 128 (the
+    library's products and the separate norm kernels of steps above 64 rows), with padding rows: 12 decode steps whose logits are the plain implementation's at every row and step, on
     scattered pages, and a page no sequence owns stays as it was (tests/test_cuda_graphs.py:20-45
     at the buckets its batch of three never reaches)."""
     from tensorline_amd.cache.manager import CacheManager
@@ -328,8 +328,8 @@ def test_graph_replay_of_wide_buckets_matches_plain(case, rows, bucket, dtype):
     page = case.page
     per_seq = max(-(-(len(p) + steps) // page) for p in case.prompts)
     cache = CacheManager(model.cache_needs(), model.schedule, model.state_needs(), page_size=page,
-                         num_blocks=rows * per_seq + 9, max_requests=64, dtype=model.dtype, device=DEV)
-    runner = GraphRunner(model, cache, max_batch=64, max_blocks_per_seq=per_seq)
+                         num_blocks=rows * per_seq + 9, max_requests=128, dtype=model.dtype, device=DEV)
+    runner = GraphRunner(model, cache, max_batch=128, max_blocks_per_seq=per_seq)
     held = cache.groups[0].allocator.take(7)                  # so that tables do not start at page 0
     bystander = held[3]
     cache.storage(0)["k"][bystander].fill_(7.0)
@@ -616,9 +616,11 @@ def test_library_tuning_keeps_results(folder_b):
     sp = SamplingParams(max_tokens=6, stop_token_ids=NO_STOP)
     plainly = LLM(d, dtype="bfloat16", device=DEV, num_blocks=64, block_size=8, max_batched_tokens=128)
     want = plainly.generate(prompt, sp)[0].token_ids
-    tuned = LLM(d, dtype="bfloat16", device=DEV, num_blocks=64, block_size=8, max_batched_tokens=128, tune_library=True)
+    # with more sequences than the engine's own kernels take rows, the graphs' row counts above that are searched too
+    tuned = LLM(d, dtype="bfloat16", device=DEV, num_blocks=64, block_size=8, max_batched_tokens=128, tune_library=True,
+                max_num_seqs=96)
     try:
-        assert tuned.model.tune_library(128) >= 1
+        assert tuned.engine.runner.batch_buckets[-1] == 96 and tuned.model.tune_library(128) >= 1
         assert tuned.generate(prompt, sp)[0].token_ids == want
     finally:
         torch.cuda.tunable.enable(False)
