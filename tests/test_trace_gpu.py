@@ -185,3 +185,42 @@ def test_trace_run_program(setup, tmp_path):
 
     got = helpers.collect_logits(run_step, steps)
     _compare(got, want, reqs, LIMIT["float32"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_massive_hidden_channels_keep_the_tolerance(name, dtype, tmp_path):
+    """Trained checkpoints have a few hidden channels tens of times larger than the rest, fed by the
+    embedding and by single rows of the down projections; random weights have none.  With two such
+    channels (x60 and x-40 in the embedding, a down-projection row x20, a norm gain x8) the residual
+    stream, the norms' sums of squares and the products that carry them must still give the plain
+    logits within the usual limits, whole and with the last tokens decoded one by one."""
+    import torch
+    from safetensors.torch import load_file, save_file
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.replay import TraceSession
+    d = helpers.make_model_dir(tmp_path, name, seed=3)
+    path = os.path.join(d, "model.safetensors")
+    t = load_file(path)
+    for k in list(t):
+        if k.endswith("embed_tokens.weight"):
+            t[k] = t[k].clone()
+            t[k][:, 3] *= 60
+            t[k][:, 17] *= -40
+        if k.endswith("down_proj.weight"):
+            t[k] = t[k].clone()
+            t[k][3] *= 20
+        if k.endswith("input_layernorm.weight"):
+            t[k] = t[k].clone()
+            t[k][17] *= 8
+    save_file(t, path, metadata={"format": "pt"})
+    w, cfg = plain.load_folder(d)
+    assert float(w["model.embed_tokens.weight"][:, 3].abs().max()) > 20 * float(w["model.embed_tokens.weight"][:, 4].abs().max())
+    reqs = {f"r{i}": p for i, p in enumerate(helpers.prompts_for(name, [3, 70, 129, 40], seed=5))}
+    want = helpers.plain_logits(w, cfg, reqs)
+    for cut in ("whole", "decode"):
+        steps = CUTS[cut](reqs)
+        model, _ = load_model(d, dtype, "cuda:0")
+        session = TraceSession(model, helpers.max_live_tokens(steps), page_size=helpers.PAGE[name])
+        worst = _compare(helpers.collect_logits(session.step, steps), want, reqs, LIMIT[dtype])
+        print(f"config {name} with massive channels, {cut}, {dtype}: worst relative error {worst:.3e}")
