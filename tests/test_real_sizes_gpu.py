@@ -126,22 +126,23 @@ def batch_decode_steps(copies: dict[str, list[int]], tail: int, budget: int = 20
     return steps
 
 
-@pytest.mark.parametrize("rows, graphs", [(8, False), (8, True), (40, False), (40, True)],
-                         ids=["8-rows-eager", "8-rows-graph", "40-rows-eager", "40-rows-graph"])
+@pytest.mark.parametrize("rows, graphs", [(8, False), (8, True), (40, False), (40, True), (72, True)],
+                         ids=["8-rows-eager", "8-rows-graph", "40-rows-eager", "40-rows-graph", "72-rows-graph"])
 def test_decoding_many_rows_at_real_layer_sizes(oracle, engine_model, rows, graphs):
-    """The last 32 tokens of 8 and of 40 requests decoded together: the few-row and the
+    """The last 32 tokens of 8, 40 and 72 requests decoded together: the few-row and the
     17-to-64-row kernels of the bfloat16 path, eagerly and replayed from the graphs of the buckets
-    of 8 and of 40 rows."""
+    of 8 and of 40 rows, and the library's products (the down projection's K in shares) inside the
+    graph of 128 rows."""
     from tensorline_amd.engine.replay import TraceSession
     d, reqs, want = oracle
     dtype, model = engine_model
     names = ["short", "mid", "long", "short", "mid"] if rows == 8 else ["short", "mid"]
-    source = {f"c{i}": ("long" if rows == 40 and i in (7, 31) else names[i % len(names)]) for i in range(rows)}
+    source = {f"c{i}": ("long" if rows >= 40 and i in (7, 31) else names[i % len(names)]) for i in range(rows)}
     copies = {rid: reqs[name] for rid, name in source.items()}
     steps = only_kept(batch_decode_steps(copies, tail=32), source.get)
     # room for 64 requests: 40 rows then replay the graph of 64 rows, 24 of them padding
-    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=PAGE, max_requests=max(rows, 64 if rows > 16 else 8),
-                           graphs=graphs)
+    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=PAGE,
+                           max_requests=128 if rows > 64 else 64 if rows > 16 else 8, graphs=graphs)
     got = helpers.collect_logits(session.step, steps)
     assert {(source[rid], p) for rid, p in got} == {k for k in want if k[0] in set(source.values())}
     worst = compare(got, want, source.get, LIMIT[dtype])
