@@ -762,6 +762,11 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         split_len, nsplit = _fit_key_splits(int(split_keys) if split_keys else GENERIC_SPLIT_KEYS, plan.max_context,
                                             plan.fit_context)
         _check(split_len % 64 == 0, "paged_attention: a split of the any-shape kernel is a multiple of 64 keys")
+        # Whether the runs go through the merge kernel is a matter of the longest context the engine
+        # runs, not of this step's: a step of short contexts and its twin in a graph captured for long
+        # ones take the same path and give the same bits (a second, empty run costs nothing).
+        if nsplit == 1 and max(plan.max_context, plan.fit_context) > split_len:
+            nsplit = 2
         if nsplit > 1:
             ws = torch.empty(T * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
     _call("tl_attention_generic", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],

@@ -311,6 +311,44 @@ def test_graph_decode_matches_eager_and_isolates_padding(folder_b):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_replayed_step_and_its_eager_twin_give_the_same_bits(name, dtype, tmp_path):
+    """Up to 16 rows a decode step replayed from a graph (padded batch, context rounded up to the
+    graph's bucket) and the same step run eagerly by a runner that knows the same longest context
+    give the same logits to the bit, with the MFMA attention kernels (B in bfloat16) and with the
+    any-shape ones (A: head size 16; B in 32-bit), whose keys go through the merge kernel in the
+    graph although these contexts would fit one run."""
+    from tensorline_amd.cache.manager import CacheManager
+    from tensorline_amd.engine.batch import StepEntry
+    from tensorline_amd.engine.graphs import GraphRunner
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.runner import ModelRunner
+    d = helpers.make_model_dir(tmp_path, name, seed=8)
+    model, _ = load_model(d, dtype, DEV)
+    page = DRIVE[name]["page"]
+    mk = lambda: CacheManager(model.cache_needs(), model.schedule, model.state_needs(), page_size=page, num_blocks=160,
+                              max_requests=8, dtype=model.dtype, device=DEV)
+    ce, cg = mk(), mk()
+    eager, graph = ModelRunner(model, ce), GraphRunner(model, cg, max_batch=8, max_blocks_per_seq=512 // page)
+    eager.fit_context = graph.fit_context
+    seqs = [list(p) for p in helpers.prompts_for(name, [2, 13, 40, 7, 90], seed=4)]
+    for c in (ce, cg):
+        for i, s in enumerate(seqs):
+            c.add_request(i)
+            assert c.grow(i, len(s) + 13)
+    first = [StepEntry(i, s, 0, [len(s) - 1]) for i, s in enumerate(seqs)]
+    le, lg = eager.step(first).clone(), graph.step(first).clone()
+    assert torch.equal(le, lg)
+    for step in range(12):
+        for s, t in zip(seqs, lg.argmax(-1).tolist()):
+            s.append(t)
+        entries = [StepEntry(i, [s[-1]], len(s) - 1, [0]) for i, s in enumerate(seqs)]
+        le, lg = eager.step(entries).clone(), graph.step(entries).clone()
+        assert torch.equal(le, lg), (step, float((le - lg).abs().max()))
+    assert graph.graph_replays == 12
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("rows, bucket", [(19, 32), (41, 64), (70, 128)])
 def test_graph_replay_of_wide_buckets_matches_plain(case, rows, bucket, dtype):
     """Graphs of 32 and of 64 rows (the 17-to-64-row kernels inside a captured graph) and of 128 (the
