@@ -70,6 +70,9 @@ class TraceSession:
             tokens = [int(t) for t in e["tokens"]]
             if not tokens:
                 raise TraceError(f"request {rid!r} brings no tokens")
+            vocab = getattr(self.model, "vocab_size", None)
+            if vocab is not None and any(t < 0 or t >= vocab for t in tokens):
+                raise TraceError(f"request {rid!r} brings a token id outside [0, {vocab})")
             if rid not in self.computed:
                 if self.cache.add_request(rid) is None:
                     raise TraceError(f"more than {self.cache.max_requests} requests are live at once (--max-requests)")

@@ -51,3 +51,13 @@ def test_more_live_requests_than_the_default_when_asked_for(setup, cpu_kernels):
     small = TraceSession(model, 64 * len(ids), page_size=16, max_requests=4)
     with pytest.raises(TraceError, match="max-requests"):
         small.step([{"id": i, "tokens": toks, "want": []} for i in ids])
+    # what a step may not bring: a token id outside the vocabulary, no tokens, a request twice, a place outside its tokens
+    fresh = TraceSession(model, 128, page_size=16)
+    for bad, word in (([{"id": "a", "tokens": [model.vocab_size], "want": []}], "token id"),
+                      ([{"id": "a", "tokens": [-1], "want": []}], "token id"),
+                      ([{"id": "a", "tokens": [], "want": []}], "no tokens"),
+                      ([{"id": "a", "tokens": [1], "want": []}, {"id": "a", "tokens": [2], "want": []}], "twice")):
+        with pytest.raises(TraceError, match=word):
+            fresh.step(bad)
+    with pytest.raises(ValueError, match="outside its 2 tokens"):
+        fresh.step([{"id": "b", "tokens": [1, 2], "want": [2]}])
