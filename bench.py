@@ -348,6 +348,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--dtype", default="bfloat16")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--prefill-behind", type=int, default=0,
+                    help="measure the prefill as a portion behind this many cached tokens (0: a fresh prompt)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-overlap", action="store_true", help="read every decode step's tokens before queueing the next")
@@ -378,7 +380,7 @@ def main() -> int:
     cfg = make_config(args.layers, args.shape)
     full_layers = SHAPES[args.shape]["num_hidden_layers"]
     max_batch = max(args.batch, 1 if args.no_points else 64)
-    max_len = args.context + 16
+    max_len = max(args.context, args.prefill_behind + args.prefill_tokens) + 16
     page = 16
     llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
               num_blocks=max_batch * (-(-max_len // page)) + 8, max_num_seqs=max_batch, max_batched_tokens=2048,
@@ -394,7 +396,10 @@ def main() -> int:
                 "ctx": round(run["mean_context"], 1), "GBps": round(gbps, 1), "hbm_frac": round(gbps / HBM_GBPS, 4)}
 
     main_run = bench_decode(llm, args.batch, args.context, args.steps, args.warmup, args.seed + 1)
-    pre = bench_prefill(llm, args.prefill_tokens, 3, args.seed + 2)
+    if args.prefill_behind > 0:
+        pre = bench_prefill_portion(llm, args.prefill_behind, args.prefill_tokens, 3, args.seed + 2)
+    else:
+        pre = bench_prefill(llm, args.prefill_tokens, 3, args.seed + 2)
     points = {}
     if not args.no_points:
         for b in (1, 64):
@@ -469,7 +474,8 @@ def main() -> int:
         torch.cuda.empty_cache()
     step_s = main_run["ms_per_step"] / 1e3
     achieved = decode_bytes(cfg, args.batch, int(main_run["mean_context"]), elem) / step_s / 1e9
-    flops = prefill_flops(cfg, args.prefill_tokens)
+    flops = (prefill_portion_flops(cfg, args.prefill_tokens, args.prefill_behind) if args.prefill_behind > 0
+             else prefill_flops(cfg, args.prefill_tokens))
     line = {
         "metric": f"decode tok/s @ batch {args.batch}, context {args.context} (Qwen2.5-{args.shape.upper()} shape)",
         "value": round(main_run["tok_s"], 1),
@@ -494,7 +500,8 @@ def main() -> int:
             "overlap": not args.no_overlap,
             "decode_graph_replays": main_run["graph_replays"], "mean_context": round(main_run["mean_context"], 1),
         },
-        "prefill": {"value": round(pre["tok_s"], 1), "tokens": args.prefill_tokens, "ms": round(pre["s"] * 1e3, 3),
+        "prefill": {"value": round(pre["tok_s"], 1), "tokens": args.prefill_tokens, "behind": args.prefill_behind,
+                    "ms": round(pre["s"] * 1e3, 3),
                     "frac": round(flops / pre["s"] / PEAK_FLOPS[dtype_key], 4),
                     "frac_of_measured_gemm": round(flops / pre["s"] / (machine["gemm_TFLOPs"] * 1e12), 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
