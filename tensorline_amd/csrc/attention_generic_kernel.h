@@ -19,8 +19,16 @@
 // in blocks of 16 keys, the softmax of the tile per row (row maximum and sum by butterflies over
 // the 16 lanes that hold a row), rescales what it has summed so far (online softmax), passes P
 // through LDS into operand layout and adds P V.  Every sum runs in an order fixed by absolute key
-// positions and by the row alone, so the result for a position depends neither on how the
-// sequence was cut into steps nor on what else is in the batch.
+// positions, by the row, and by which of three forms the launch takes: rows of prompt portions (a
+// wave per 16 rows, a tile's keys in order); a step in which no sequence brings more than one
+// token, unsplit (the four waves share the rows and take a block of 16 keys of each tile each,
+// put together at the end in the order of the waves); and that step with the keys split into runs
+// at absolute positions, added by the merge kernel in ascending order.  The form follows from the
+// step (its longest query, whether it only decodes) and from the engine's longest context, never
+// from the context of one sequence.  Within a form the result for a position depends neither on
+// how the sequence was cut into steps nor on what else is in the batch, to the bit, and a step
+// replayed from a graph takes the form of its eager twin; between forms (a token decoded alone,
+// or beside another request's prompt portion) results agree within float rounding.
 //
 // Operand layout of the 16x16x4 product D = A B + C: lane l gives A[l % 16][l / 16] and
 // B[l / 16][l % 16]; it holds D[4 (l / 16) + v][l % 16] in register v.  The four k of one product

@@ -3,7 +3,9 @@
 A step takes, per request, its next tokens: a whole prompt, a portion of one cut anywhere, or a
 single decoded token, in any mix (reference: ``SeqChunk`` and the flattening in
 tensorline/paged.py:100-106,194-238).  All index data of a step is packed into one int32 vector
-and copied to the device once; the kernels read views of it.
+and copied to the device once; the kernels read views of it.  Nothing here knows what a mixer
+caches or how it launches its kernels: a part that wants an index list of its own on the device
+computes it from the step's facts (``step_vectors``) and finds it in ``StepContext.extra``.
 """
 from __future__ import annotations
 
@@ -26,19 +28,17 @@ class StepEntry:
 
 
 @dataclass
-class AttentionPlan:
-    """Host-side facts about the step that attention kernels choose their launch shape from."""
+class StepFacts:
+    """What the host knows about the step's shape.  Parts choose their launches from it; nothing in
+    it belongs to one kind of part."""
     max_context: int = 0          # largest start + len over the step's sequences
     max_query_len: int = 0        # largest number of tokens one sequence brings
     decode_only: bool = False     # every sequence brings exactly one token
-    num_seqs: int = 0
-    q_lens: list[int] = field(default_factory=list)
-    starts: list[int] = field(default_factory=list)
-    # In a step that mixes prompt portions with one-token sequences: the indices of the latter
-    # (also on the device, ``StepContext.single_seqs``), so that they can be given to a kernel of their own.
-    singles: list[int] = field(default_factory=list)
+    num_seqs: int = 0             # sequences of the step, padding sequences (one token each, after the real ones) included
+    q_lens: list[int] = field(default_factory=list)    # tokens each real sequence brings
+    starts: list[int] = field(default_factory=list)    # tokens each real sequence has cached already
     # The longest context the engine will ever run, if the caller knows it (0: unknown).  Choices
-    # that must be the same in every step of an engine (the length of a key split) are made for it.
+    # that must be the same in every step of an engine are made for it.
     fit_context: int = 0
 
 
@@ -50,14 +50,6 @@ class LayerCache:
     tables: torch.Tensor | None       # int32 [S, NB]: page ids of each sequence
     write: bool                       # False: the entry reads a cache another entry wrote
     state: torch.Tensor | None = None  # [slots + 1, *shape] fixed-size per-request state, if any
-
-    @property
-    def k(self) -> torch.Tensor | None:
-        return self.planes.get("k")
-
-    @property
-    def v(self) -> torch.Tensor | None:
-        return self.planes.get("v")
 
 
 @dataclass
@@ -71,8 +63,9 @@ class StepContext:
     ctx_start: torch.Tensor           # int32 [S]: tokens of the sequence already cached
     state_slots: torch.Tensor         # int32 [S]
     logit_rows: torch.Tensor          # int32 [R]
-    attention_plan: AttentionPlan
-    single_seqs: torch.Tensor | None = None   # int32 [len(attention_plan.singles)], if there are any
+    facts: StepFacts
+    # int32 vectors that parts asked to have uploaded with the step (``step_vectors``), by name
+    extra: dict[str, torch.Tensor] = field(default_factory=dict)
     # host mirrors, for parts that loop over sequences on the host
     host_q_start: list[int] = field(default_factory=list)
     host_ctx_start: list[int] = field(default_factory=list)
@@ -89,7 +82,7 @@ class PackedBatch:
     R: int
     offsets: dict[str, tuple[int, int]]
     group_nb: list[int]
-    plan: AttentionPlan
+    facts: StepFacts
     host_q_start: list[int]
     host_ctx_start: list[int]
     host_state_slots: list[int]
@@ -99,10 +92,12 @@ class PackedBatch:
 def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[int]]], state_slots: Sequence[int],
                page_size: int, num_groups: int, scratch_page: int, vocab_size: int,
                pad_seqs: int = 0, pad_nb: Sequence[int] | None = None, scratch_slot: int = 0,
-               windowed: Sequence[bool] | None = None) -> PackedBatch:
+               windowed: Sequence[bool] | None = None, vectors=None) -> PackedBatch:
     """Flatten a step.  ``tables[s][g]`` is the page table of sequence ``s`` in group ``g`` and must
     cover positions < start + len.  With ``pad_seqs``/``pad_nb`` the batch is padded to a fixed
-    shape with one-token rows that touch only the scratch page and the scratch slot."""
+    shape with one-token rows that touch only the scratch page and the scratch slot.
+    ``vectors``: a function from the step's :class:`StepFacts` to int32 vectors by name (index lists
+    that parts want on the device for this step); they travel in the same upload."""
     S = len(entries)
     if S == 0:
         raise ValueError("a step needs at least one entry")
@@ -196,9 +191,13 @@ def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[
     pieces: list[tuple[str, np.ndarray]] = [
         ("ids", ids), ("pos", pos), ("seq_of_token", seq_of), ("q_start", q_start), ("ctx_start", ctx_start),
         ("state_slots", slots_state), ("logit_rows", np.asarray(rows, np.int32))]
-    decode_only = all(n == 1 for n in q_lens)
-    singles = [] if decode_only else [s for s, n in enumerate(q_lens) if n == 1] + list(range(S, S_pad))
-    pieces.append(("single_seqs", np.asarray(singles, np.int32)))
+    starts = [e.start for e in entries]
+    facts = StepFacts(
+        max_context=max(st + n for st, n in zip(starts, q_lens)), max_query_len=max(q_lens),
+        decode_only=all(n == 1 for n in q_lens), num_seqs=S_pad, q_lens=q_lens, starts=starts)
+    extra = vectors(facts) if vectors is not None else {}
+    for name in sorted(extra):
+        pieces.append(("extra:" + name, np.asarray(extra[name], np.int32).reshape(-1)))
     for g in range(num_groups):
         pieces.append((f"slots{g}", g_slots[g]))
         pieces.append((f"tables{g}", g_tables[g].reshape(-1)))
@@ -207,10 +206,6 @@ def pack_batch(entries: Sequence[StepEntry], tables: Sequence[Sequence[Sequence[
         offsets[name] = (off, arr.size)
         off += arr.size
     data = np.concatenate([a for _, a in pieces]) if off else np.zeros(0, np.int32)
-    starts = [e.start for e in entries]
-    plan = AttentionPlan(
-        max_context=max(st + n for st, n in zip(starts, q_lens)), max_query_len=max(q_lens),
-        decode_only=decode_only, num_seqs=S_pad, q_lens=q_lens, starts=starts, singles=singles)
-    return PackedBatch(data.astype(np.int32, copy=False), T, S_pad, len(rows), offsets, group_nb, plan,
+    return PackedBatch(data.astype(np.int32, copy=False), T, S_pad, len(rows), offsets, group_nb, facts,
                        [int(v) for v in q_start], [int(v) for v in ctx_start], [int(v) for v in slots_state],
                        logits_for_all_rows=rows == list(range(T)))

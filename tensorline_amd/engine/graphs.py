@@ -92,14 +92,14 @@ class GraphRunner(ModelRunner):
         tables = [[[cache.scratch_page] for _ in range(ng)]]
         packed = pack_batch([pad], tables, [cache.scratch_slot], cache.page_size, ng, cache.scratch_page,
                             self.model.vocab_size, pad_seqs=B, pad_nb=[self.max_blocks] * ng,
-                            scratch_slot=cache.scratch_slot)
+                            scratch_slot=cache.scratch_slot, vectors=self._vectors)
         return packed
 
     @torch.inference_mode()
     def _capture(self, B: int, C: int) -> _Captured:
         packed = self._padding_batch(B)
-        packed.plan.max_context, packed.plan.fit_context = C, self.fit_context
-        packed.plan.decode_only = True
+        packed.facts.max_context, packed.facts.fit_context = C, self.fit_context
+        packed.facts.decode_only = True
         n = packed.data.size
         dev = torch.empty(n, dtype=torch.int32, device=self.device)
         host = torch.empty(n, dtype=torch.int32, pin_memory=True)

@@ -52,6 +52,12 @@ class ModelRunner:
             self._dev[:n].copy_(self._host[:n])
         return self._dev
 
+    def _vectors(self, facts) -> dict:
+        """Index vectors the model's parts want uploaded with this step; they see the engine's longest context."""
+        facts.fit_context = self.fit_context
+        fn = getattr(self.model, "step_vectors", None)
+        return fn(facts) if fn is not None else {}
+
     def pack(self, entries: Sequence[StepEntry], pad_seqs: int = 0, pad_nb: Sequence[int] | None = None) -> PackedBatch:
         cache = self.cache
         ngroups = len(cache.groups)
@@ -59,8 +65,8 @@ class ModelRunner:
         slots = [cache.state_slot(e.rid) for e in entries]
         packed = pack_batch(entries, tables, slots, cache.page_size, ngroups, cache.scratch_page,
                             self.model.vocab_size, pad_seqs=pad_seqs, pad_nb=pad_nb, scratch_slot=cache.scratch_slot,
-                            windowed=[g.window > 0 for g in cache.groups])
-        packed.plan.fit_context = self.fit_context
+                            windowed=[g.window > 0 for g in cache.groups], vectors=self._vectors)
+        packed.facts.fit_context = self.fit_context
         return packed
 
     def context(self, packed: PackedBatch, dev: torch.Tensor) -> tuple[StepContext, list[LayerCache]]:
@@ -71,10 +77,10 @@ class ModelRunner:
         ctx = StepContext(
             num_tokens=packed.T, num_seqs=packed.S, ids=view("ids"), pos=view("pos"),
             seq_of_token=view("seq_of_token"), q_start=view("q_start"), ctx_start=view("ctx_start"),
-            state_slots=view("state_slots"), logit_rows=view("logit_rows"), attention_plan=packed.plan,
+            state_slots=view("state_slots"), logit_rows=view("logit_rows"), facts=packed.facts,
             host_q_start=packed.host_q_start, host_ctx_start=packed.host_ctx_start,
             host_state_slots=packed.host_state_slots, logits_for_all_rows=packed.logits_for_all_rows,
-            single_seqs=view("single_seqs") if packed.plan.singles else None)
+            extra={name[6:]: view(name) for name in packed.offsets if name.startswith("extra:")})
         cache = self.cache
         g_slots = [view(f"slots{g}") for g in range(len(cache.groups))]
         g_tables = [view(f"tables{g}").view(packed.S, packed.group_nb[g]) for g in range(len(cache.groups))]

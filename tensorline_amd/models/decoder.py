@@ -37,6 +37,7 @@ class DecoderModel:
         self.final_norm = build_part("norm", spec.final_norm, layer_prefix="", **common)
         self.head = build_part("head", spec.head, layer_prefix="", vocab_size=spec.vocab_size, **common)
         self._after: list[Intake | None] | None = None     # per schedule entry: what its successor takes
+        self._vector_makers: list | None = None
 
     def _all_parts(self):
         yield self.embedding
@@ -115,6 +116,21 @@ class DecoderModel:
         intakes = [b.intake() if hasattr(b, "intake") else Intake() for b in takers[1:]] + [self._tail_intake()]
         return [nxt if hasattr(b, "intake") else None for b, nxt in zip(takers, intakes)]
 
+    def step_vectors(self, facts) -> dict:
+        """int32 index vectors that parts want on the device for a step of this shape, by name.  A
+        part that has ``step_vectors(facts) -> {name: vector}`` is asked; parts of one class share
+        their vectors, so one of them answers for all.  They are found in ``StepContext.extra``."""
+        if self._vector_makers is None:
+            seen = {}
+            for p in self._all_parts():
+                if hasattr(p, "step_vectors"):
+                    seen.setdefault(type(p), p)
+            self._vector_makers = list(seen.values())
+        out: dict = {}
+        for p in self._vector_makers:
+            out.update(p.step_vectors(facts))
+        return out
+
     def forward(self, ctx, caches) -> torch.Tensor:
         """``caches[i]`` is the view of the cache for schedule entry ``i``."""
         if self._after is None:
@@ -130,7 +146,9 @@ class DecoderModel:
         if ctx.logit_rows.numel() == 0:
             # the residual stream is complete only after the last add; nothing reads it here
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=x.device)
-        if isinstance(carry, kernels.NormedRows):
+        if getattr(carry, "stands_for_normed_rows", False):
+            # the last block's carry already is the final norm's output in the form the head takes
+            # (negotiated by ``_tail_intake``); the carry knows how to give the wanted rows of itself
             h = carry if ctx.logits_for_all_rows else carry.take(ctx.logit_rows)
         else:
             h = self.final_norm.forward(x, carry, rows=ctx.logit_rows)

@@ -206,6 +206,7 @@ class NormedRows:
     sumsq: torch.Tensor
     dim: int
     eps: float
+    stands_for_normed_rows = True      # a carry of this form is a norm's output; ``take`` picks rows of it
 
     def take(self, index: torch.Tensor) -> "NormedRows":
         """The rows ``index`` (int tensor) only."""
@@ -596,6 +597,14 @@ def rope_store(qkv: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor | No
           k_cache.shape[1] if write else 0, _ptr(bias), _stream())
 
 
+def one_token_sequences(facts) -> list[int]:
+    """The sequences that bring one token to a step that also holds prompt portions (padding
+    sequences among them); none in a step of one token per sequence."""
+    if facts.decode_only:
+        return []
+    return [s for s, n in enumerate(facts.q_lens) if n == 1] + list(range(len(facts.q_lens), facts.num_seqs))
+
+
 def _singles_get_own_launch(plan, singles: list[int], num_heads: int, num_kv_heads: int, head_dim: int,
                             window: int) -> bool:
     """Whether the one-token sequences of a step with prompt portions are worth a launch of their
@@ -660,7 +669,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     """Causal attention of each token over the cached keys of its sequence.
 
     ``q``: [T, >= nq*d] with the query heads in the first nq*d columns (row stride free);
-    ``tables``: int32 [S, NB] page ids; ``seq_of_token``, ``pos``: int32 [T].  ``window`` > 0
+    ``tables``: int32 [S, NB] page ids; ``seq_of_token``, ``pos``: int32 [T]; ``plan``: the step's
+    host-side facts (``max_context``, ``max_query_len``, ``decode_only``, ``num_seqs``, ``q_lens``,
+    ``starts``, ``fit_context``).  ``window`` > 0
     limits a token at position p to keys [p - window + 1, p].  Returns [T, nq*d].
 
     bfloat16 with a head size of 32, 64 or 128 and pages of a multiple of 8 tokens runs on the
@@ -672,7 +683,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
     A step with prompt portions does not split keys: its one-token sequences would each be walked
     by one work-group from the first key to the last.  With ``single_seqs`` (int32, the indices
-    ``plan.singles`` on the device) they are computed by a launch of their own where that is
+    ``one_token_sequences(plan)`` on the device) they are computed by a launch of their own where that is
     estimated to be faster (``_singles_get_own_launch``), split like a decode step of that many
     sequences, and the launch for the portions leaves them out.  ``route_singles`` forces that
     on or off."""
@@ -700,7 +711,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _i32(ctx_start, "ctx_start", S)
         G = num_heads // num_kv_heads
         skip_single = 0
-        singles = plan.singles if single_seqs is not None and not plan.decode_only and split_keys is None else []
+        singles = one_token_sequences(plan) if single_seqs is not None and split_keys is None else []
         if singles and route_singles is not False:
             _i32(single_seqs, "single_seqs", len(singles))
             ctx1 = max([plan.starts[s] + 1 for s in singles if s < len(plan.starts)] + [1])
@@ -753,6 +764,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         q_start = torch.zeros(S + 1, dtype=torch.int32, device=q.device)
         q_start[1:] = torch.cumsum(counts, 0)
         max_query_len = int(counts.max().item()) if T else 1
+        # a row of a sequence the table does not have would be computed by nobody and merged from nothing
+        _check(int(counts.sum().item()) == T, f"paged_attention: seq_of_token names sequences outside the {S} of the page table")
     _check(attention_takes_head_dim(head_dim), f"paged_attention: head size {head_dim} must be a multiple of 16, at most 256")
     # Steps of one token per sequence split the keys into runs of GENERIC_SPLIT_KEYS at absolute positions
     # (longer runs only where the longest context the engine ever runs would need more splits than a launch

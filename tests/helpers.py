@@ -153,19 +153,35 @@ class ForcedSampler:
     tokens given for it (a request is known by its seed), and the logits it was shown are kept.
     With the plain implementation's own tokens forced, a bfloat16 run sees the contexts the
     plain run saw at every position, so its logits can be compared one by one; a token picked
-    from near-equal logits cannot send the rest of the comparison elsewhere."""
+    from near-equal logits cannot send the rest of the comparison elsewhere.
+
+    It has both of the sampler's forms.  ``sample_device`` awaits nothing: it keeps a copy of the
+    logits on the device (a replayed graph writes the next step's over them) and returns the forced
+    tokens as an int32 tensor on the device, so the engine leaves decode steps in flight and takes
+    the next step's token ids from the device, as it does in serving."""
 
     def __init__(self, forced: dict[int, list[int]]):
         self.forced = forced
-        self.logits: dict[tuple[int, int], np.ndarray] = {}       # (seed, index of the generated token) -> row
+        self._rows: dict[tuple[int, int], np.ndarray] = {}        # (seed, index of the generated token) -> row
+        self._kept: list = []                                      # (logits on the device, seeds, indices), not read yet
+
+    @property
+    def logits(self) -> dict[tuple[int, int], np.ndarray]:
+        for dev, seeds, indices in self._kept:
+            for row, seed, index in zip(dev.cpu().numpy(), seeds, indices):
+                self._rows[(seed, index)] = row
+        self._kept.clear()
+        return self._rows
+
+    def sample_device(self, logits, temperatures, top_ps, seeds, indices):
+        self._kept.append((logits.detach().to(torch.float32, copy=True), list(seeds), list(indices)))
+        # a row past a request's last forced token is one the engine throws away (the step queued ahead of a stop)
+        toks = torch.tensor([self.forced[s][i] if i < len(self.forced[s]) else 0 for s, i in zip(seeds, indices)],
+                            dtype=torch.int32)
+        return toks.to(logits.device)
 
     def sample(self, logits, temperatures, top_ps, seeds, indices):
-        rows = logits.to(torch.float32).cpu().numpy()
-        out = []
-        for row, seed, index in zip(rows, seeds, indices):
-            self.logits[(seed, index)] = row.copy()
-            out.append(self.forced[seed][index])
-        return out
+        return self.sample_device(logits, temperatures, top_ps, seeds, indices).tolist()
 
 
 def watch_pages(cache) -> dict:

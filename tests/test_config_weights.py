@@ -56,16 +56,21 @@ def test_registry(tmp_path):
     assert len(spec.layers) == 2 and spec.layers[1].mixer.params["num_heads"] == 6
 
 
-@pytest.mark.parametrize("head_dim", [8, 40, 272])
+@pytest.mark.parametrize("head_dim", [272, 300])
 def test_head_sizes_no_kernel_serves_are_refused_when_the_model_is_built(head_dim):
     """The configuration allows any even head size; the attention part refuses, before any weight is
-    read, those the kernels do not take, instead of failing in the first step."""
+    read, those the kernels do not take, instead of failing in the first step.  Sizes between the
+    kernels' steps of 16 are served at the next step, with zeros added to every head at loading."""
     from tensorline_amd.models.decoder import DecoderModel
     arch = get_architecture("Qwen2ForCausalLM")
     spec = arch.build_spec(Qwen2Config.from_dict(dict(BASE, head_dim=head_dim)))
     with pytest.raises(ValueError, match=f"head size of {head_dim}"):
         DecoderModel(spec, torch.float32, "cpu")
-    DecoderModel(arch.build_spec(Qwen2Config.from_dict(dict(BASE, head_dim=48))), torch.float32, "cpu")
+    for d, served_at in ((48, 48), (8, 16), (40, 48), (250, 256)):
+        model = DecoderModel(arch.build_spec(Qwen2Config.from_dict(dict(BASE, head_dim=d))), torch.float32, "cpu")
+        mixer = model.blocks[0].mixer
+        assert (mixer.head_dim, mixer.kernel_dim) == (d, served_at)
+        assert model.cache_needs()[0].planes[0].shape[-1] == served_at       # the cache is laid out for the kernels' size
 
 
 def test_engine_config_names():

@@ -42,7 +42,7 @@ class Case:
                 "portions": dict(graphs=True, max_batched_tokens=d["chunk"]),
                 "preemption": dict(graphs=False, num_blocks=d["tight_blocks"], prefix_caching=False),
                 "preemption-shared-prefixes": dict(graphs=True, num_blocks=d["tight_blocks"], prefix_caching=True),
-                "seq-limit": dict(graphs=True, max_num_seqs=2)}
+                "seq-limit": dict(graphs=True, max_num_seqs=2), "graphs-no-overlap": dict(graphs=True, overlap=False)}
 
 
 @pytest.fixture(scope="module", params=["A", "B"])
@@ -64,7 +64,7 @@ def greedy_want(folder_b):
     return prompts, [plain.greedy_generate(w, cfg, p, 24) for p in prompts]
 
 
-REGIMES = ["eager", "graphs", "portions", "preemption", "preemption-shared-prefixes", "seq-limit"]
+REGIMES = ["eager", "graphs", "portions", "preemption", "preemption-shared-prefixes", "seq-limit", "graphs-no-overlap"]
 
 
 @pytest.mark.parametrize("regime", REGIMES)
@@ -92,7 +92,9 @@ def test_greedy_generation_matches_plain(case, regime):
 def test_bfloat16_logits_through_the_scheduler_match_plain(case, regime):
     """bfloat16 under the scheduler, in every regime: the plain implementation's tokens are forced
     on every request, so each step sees the contexts the plain run saw, and the logits the sampler
-    is shown must be the plain ones within the bfloat16 limit at every generated position."""
+    is shown must be the plain ones within the bfloat16 limit at every generated position.  The
+    forced tokens come back on the device, so steady decoding runs as it does in serving: a step
+    queued behind the one in flight, its token ids taken from the device (graph replay, bfloat16)."""
     from tensorline_amd import SamplingParams
     opts = case.regimes()[regime]
     llm = case.llm("bfloat16", **opts)
@@ -114,6 +116,10 @@ def test_bfloat16_logits_through_the_scheduler_match_plain(case, regime):
         assert c["preemptions"] > 0
     if opts.get("graphs"):
         assert c["graph_replays"] > 0
+    if regime in ("eager", "graphs", "seq-limit"):
+        assert c["overlapped_steps"] > 0, "no decode step was queued behind the one in flight"
+    if opts.get("overlap") is False:
+        assert c["overlapped_steps"] == 0
 
 
 @pytest.mark.parametrize("block_size", [16, 32, 64, 128])

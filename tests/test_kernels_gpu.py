@@ -372,9 +372,11 @@ def test_product_adds_into_the_residual_and_prepares_the_next_norm(M, N, Kd):
 
 
 def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, spike=False, path=None, split_keys=None,
-                    route_singles=None, pool_pages=None):
+                    route_singles=None, pool_pages=None, spike_at=None):
     """Sequences of context ``lens``; the last ``q_lens[i]`` positions of each are queries.
-    pool_pages: the sequences' pages are the last ones of a pool of that many."""
+    pool_pages: the sequences' pages are the last ones of a pool of that many.  ``spike``: the key
+    at position 1 (or at ``spike_at(position of the query)``, if that is a key at all) is made to
+    match its query, so that it dominates the sum if it is seen."""
     torch.manual_seed(seed)
     S = len(lens)
     q_lens = q_lens or [1] * S
@@ -402,18 +404,21 @@ def _attention_case(dtype, nq, nkv, d, bs, lens, q_lens=None, window=0, seed=0, 
         for t in range(T):
             s = seq_of[t]
             far = 1 if lens[s] > 2 else 0
+            if spike_at is not None:
+                far = spike_at(pos[t])
+                if not 0 <= far < lens[s]:
+                    continue
             row = int(tables[s, far // bs]) * bs + far % bs
             kflat[row] = (q[t].view(nq, d)[:nkv].float() * 4).to(dtype)
-    from tensorline_amd.engine.batch import AttentionPlan
+    from tensorline_amd.engine.batch import StepFacts
     qs = [0]
     for ql in q_lens:
         qs.append(qs[-1] + ql)
-    plan = AttentionPlan(max_context=max(lens), max_query_len=max(q_lens), decode_only=max(q_lens) == 1,
-                         num_seqs=S, q_lens=list(q_lens), starts=[n - ql for n, ql in zip(lens, q_lens)])
+    plan = StepFacts(max_context=max(lens), max_query_len=max(q_lens), decode_only=max(q_lens) == 1,
+                     num_seqs=S, q_lens=list(q_lens), starts=[n - ql for n, ql in zip(lens, q_lens)])
     single_seqs = None
-    if not plan.decode_only and 1 in q_lens:
-        plan.singles = [s for s, ql in enumerate(q_lens) if ql == 1]
-        single_seqs = torch.tensor(plan.singles, dtype=torch.int32, device=DEV)
+    if K().one_token_sequences(plan):
+        single_seqs = torch.tensor(K().one_token_sequences(plan), dtype=torch.int32, device=DEV)
     out = K().paged_attention(q, kc, vc, tables, torch.tensor(seq_of, dtype=torch.int32, device=DEV),
                               torch.tensor(pos, dtype=torch.int32, device=DEV), nq, nkv, d, d ** -0.5, window=window,
                               q_start=torch.tensor(qs, dtype=torch.int32, device=DEV),
@@ -532,6 +537,25 @@ def test_attention_any_shape_kernel_splits_keys_in_one_token_steps(dtype, lens, 
     waves have a key block).  0: no split, the same kernel walking all keys."""
     got, want = _attention_case(dtype, 6, 2, d, bs, lens, None, spike=True, seed=11, path="generic", split_keys=split)
     torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 100, 101, 300])
+@pytest.mark.parametrize("split", [None, 64])
+def test_attention_any_shape_kernel_window_with_split_keys(dtype, window, split):
+    """A window in steps of one token per sequence on the any-shape kernel, where the keys are split
+    into runs: the window's first key inside a run (700 keys, window 100: key 600 of the run from
+    512), exactly on a run's edge (357 keys, window 101: key 256), whole leading runs empty, a
+    window longer than the context.  The key just outside the window matches its query: seen, it
+    would carry the sum."""
+    lens = [700, 257, 256, 9, 357]
+    got, want = _attention_case(dtype, 6, 2, 32, 8, lens, None, window=window, seed=21, spike=True, path="generic",
+                                split_keys=split, spike_at=lambda p: p - window)
+    torch.testing.assert_close(got, want, **tol(dtype, 3e-5, 2e-2))
+    inside, _ = _attention_case(dtype, 6, 2, 32, 8, lens, None, window=window, seed=21, spike=True, path="generic",
+                                split_keys=split, spike_at=lambda p: p - window + 1)
+    if window > 1:
+        assert not torch.allclose(inside, got, atol=1e-3)      # the same key one place further in is seen, and shows
 
 
 @pytest.mark.parametrize("d,bs", [(128, 8), (128, 16), (128, 32), (128, 64), (128, 128), (128, 24), (64, 8), (64, 16),

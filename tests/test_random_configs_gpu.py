@@ -66,11 +66,13 @@ def test_random_configuration_matches_plain(seed):
 
 
 @pytest.mark.parametrize("hidden,inter,vocab,d", [(50, 90, 97, 16), (7, 9, 11, 16), (100, 25, 33, 48), (1, 1, 2, 16),
-                                                  (136, 88, 300, 160), (72, 176, 777, 256)])
+                                                  (136, 88, 300, 160), (72, 176, 777, 256),
+                                                  (64, 96, 200, 8), (96, 64, 301, 40), (128, 176, 500, 72), (80, 112, 150, 120)])
 @pytest.mark.parametrize("cut", sorted(CUTS))
 def test_odd_widths_and_large_heads_match_plain(hidden, inter, vocab, d, cut):
     """Widths that are no multiple of 8 (rows of the weights are not 16-byte aligned, so no streaming
-    kernel takes them), down to a width of one, and head sizes above 128 through the whole model."""
+    kernel takes them), down to a width of one, head sizes above 128, and head sizes between the
+    kernels' steps of 16 (8, 40, 72, 120: served with zeros added to every head) through the whole model."""
     rng = random.Random(hidden * 1000 + d)
     nkv = rng.choice([1, 2, 3])
     cfg_dict = dict(architectures=["Qwen2ForCausalLM"], vocab_size=vocab, hidden_size=hidden, intermediate_size=inter,

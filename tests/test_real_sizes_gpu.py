@@ -1,9 +1,13 @@
-"""A model with the layer sizes of Qwen2.5-7B (hidden 3584, 28 query and 4 key/value heads of 128,
-feed-forward 18944, vocabulary 152064) and 2 of its 28 layers, against the plain implementation:
-the branches that only real sizes take (the wide head, products cut into shares of K, groups of
-seven query heads, hundreds of column groups in prompt attention, the 17-to-64-row kernels and
-graph buckets above 16 rows) as a whole model, in 32-bit and in bfloat16, in every way of cutting
-(analogue of the reference's tests/test_batching.py:48-64 at a size its own tests never reach)."""
+"""Models with the layer sizes of Qwen2.5-7B (hidden 3584, 28 query and 4 key/value heads of 128,
+feed-forward 18944, vocabulary 152064; 2 of its 28 layers), of Qwen2.5-14B (hidden 5120, 40 and 8
+heads, feed-forward 13824; 1 of its 48 layers) and of Qwen2.5-32B (the same with a feed-forward of
+27648; 1 of its 64 layers) against the plain implementation: the branches that only real sizes
+take (the wide head, products cut into shares of K, groups of seven and of five query heads, 224
+and 320 column tiles for 256 CUs, hundreds of column groups in prompt attention, the 17-to-64-row
+kernels and graph buckets above 16 rows) as a whole model, in 32-bit and in bfloat16 (analogue of
+the reference's tests/test_batching.py:48-64 at sizes its own tests never reach).  The 7B sizes
+run every way of cutting; the two wider shapes run whole prompts, prompt then decoding, and 8 and
+40 rows decoding from graphs."""
 import random
 
 import numpy as np
@@ -14,10 +18,15 @@ from tests import helpers, plain
 
 pytestmark = pytest.mark.gpu
 
-SHAPE_7B_2_LAYERS = dict(
+SHAPE_7B = dict(
     architectures=["Qwen2ForCausalLM"], vocab_size=152064, hidden_size=3584, intermediate_size=18944,
     num_hidden_layers=2, num_attention_heads=28, num_key_value_heads=4, head_dim=128, rope_theta=1000000.0,
     rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768)
+SHAPE_14B = dict(SHAPE_7B, hidden_size=5120, intermediate_size=13824, num_hidden_layers=1, num_attention_heads=40,
+                 num_key_value_heads=8, rms_norm_eps=1e-5)
+SHAPE_32B = dict(SHAPE_14B, intermediate_size=27648, rms_norm_eps=1e-6)
+SHAPES = {"7b-2-of-28-layers": SHAPE_7B, "14b-1-of-48-layers": SHAPE_14B, "32b-1-of-64-layers": SHAPE_32B}
+S7, S14, S32 = SHAPES
 LENGTHS = {"tiny": 3, "short": 70, "mid": 200, "long": 2100}
 LIMIT = {"float32": 1e-5, "bfloat16": 2e-2}
 PAGE = 16
@@ -33,11 +42,12 @@ def kept_positions(n: int) -> list[int]:
     return sorted(p for p in keep if p < n)
 
 
-@pytest.fixture(scope="module")
-def oracle(tmp_path_factory):
+def build_oracle(shape: str, folder: str):
+    """The model folder of a shape, requests, and the plain implementation's logits at the kept positions."""
     from tensorline_amd.config import Qwen2Config
     from tensorline_amd.weights import write_random_model
-    d = write_random_model(Qwen2Config.from_dict(SHAPE_7B_2_LAYERS), str(tmp_path_factory.mktemp("real_sizes")), seed=17)
+    print(f"real sizes: writing and running the plain model of {shape}", flush=True)
+    d = write_random_model(Qwen2Config.from_dict(SHAPES[shape]), folder, seed=17)
     w, cfg = plain.load_folder(d)
     rng = random.Random(23)
     reqs = {name: [rng.randrange(cfg["vocab_size"]) for _ in range(n)] for name, n in LENGTHS.items()}
@@ -49,16 +59,34 @@ def oracle(tmp_path_factory):
                 want[(name, p)] = logits[p].numpy().copy()
             del logits
     del w
-    return d, reqs, want
+    return d, reqs, want, {}
 
 
-@pytest.fixture(scope="module", params=["float32", "bfloat16"])
-def engine_model(request, oracle):
-    from tensorline_amd.engine.loading import load_model
-    model, _ = load_model(oracle[0], request.param, "cuda:0")
-    yield request.param, model
-    del model
+@pytest.fixture(scope="module")
+def oracles(tmp_path_factory):
+    """``oracles(shape)``: built at the first call for a shape and kept until the module's tests are
+    through, whatever order they run in (three folders of a few gigabytes, six models on the GPU)."""
+    import shutil
+    built = {}
+
+    def get(shape):
+        if shape not in built:
+            built[shape] = build_oracle(shape, str(tmp_path_factory.mktemp("real_sizes")))
+        return built[shape]
+    yield get
+    for d, _, _, models in built.values():
+        models.clear()
+        shutil.rmtree(d, ignore_errors=True)
     torch.cuda.empty_cache()
+
+
+def model_of(oracle, dtype: str):
+    """The engine's model of the shape in one dtype, loaded once."""
+    from tensorline_amd.engine.loading import load_model
+    models = oracle[3]
+    if dtype not in models:
+        models[dtype] = load_model(oracle[0], dtype, "cuda:0")[0]
+    return models[dtype]
 
 
 def only_kept(steps, source_of=lambda rid: rid):
@@ -94,17 +122,18 @@ CUTS = {"whole": helpers.steps_whole, "decode": helpers.steps_prefill_then_decod
         "mixed": lambda reqs: helpers.steps_mixed(reqs, seed=3, tail=12)}
 
 
-@pytest.mark.parametrize("cut", list(CUTS))
-def test_cuttings_match_plain_at_real_layer_sizes(oracle, engine_model, cut):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape, cut", [(S7, c) for c in CUTS] + [(s, c) for s in (S14, S32) for c in ("whole", "decode")])
+def test_cuttings_match_plain_at_real_layer_sizes(oracles, shape, cut, dtype):
     from tensorline_amd.engine.replay import TraceSession
-    d, reqs, want = oracle
-    dtype, model = engine_model
+    d, reqs, want, _ = oracle = oracles(shape)
+    model = model_of(oracle, dtype)
     steps = only_kept(CUTS[cut](reqs))
     session = TraceSession(model, helpers.max_live_tokens(steps), page_size=PAGE)
     got = helpers.collect_logits(session.step, steps)
     assert set(got) == set(want)
     worst = compare(got, want, limit=LIMIT[dtype])
-    print(f"7B layer sizes, 2 layers, {cut} {dtype}: worst relative error {worst:.3e}")
+    print(f"real layer sizes, {cut} {dtype}: worst relative error {worst:.3e}")
     assert session.cache.all_free()
 
 
@@ -126,16 +155,19 @@ def batch_decode_steps(copies: dict[str, list[int]], tail: int, budget: int = 20
     return steps
 
 
-@pytest.mark.parametrize("rows, graphs", [(8, False), (8, True), (40, False), (40, True), (72, True)],
-                         ids=["8-rows-eager", "8-rows-graph", "40-rows-eager", "40-rows-graph", "72-rows-graph"])
-def test_decoding_many_rows_at_real_layer_sizes(oracle, engine_model, rows, graphs):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize(
+    "shape, rows, graphs",
+    [(S7, 8, False), (S7, 8, True), (S7, 40, False), (S7, 40, True), (S7, 72, True)]
+    + [(s, rows, True) for s in (S14, S32) for rows in (8, 40)])
+def test_decoding_many_rows_at_real_layer_sizes(oracles, shape, rows, graphs, dtype):
     """The last 32 tokens of 8, 40 and 72 requests decoded together: the few-row and the
     17-to-64-row kernels of the bfloat16 path, eagerly and replayed from the graphs of the buckets
     of 8 and of 40 rows, and the library's products (the down projection's K in shares) inside the
     graph of 128 rows."""
     from tensorline_amd.engine.replay import TraceSession
-    d, reqs, want = oracle
-    dtype, model = engine_model
+    d, reqs, want, _ = oracle = oracles(shape)
+    model = model_of(oracle, dtype)
     names = ["short", "mid", "long", "short", "mid"] if rows == 8 else ["short", "mid"]
     source = {f"c{i}": ("long" if rows >= 40 and i in (7, 31) else names[i % len(names)]) for i in range(rows)}
     copies = {rid: reqs[name] for rid, name in source.items()}
@@ -146,9 +178,27 @@ def test_decoding_many_rows_at_real_layer_sizes(oracle, engine_model, rows, grap
     got = helpers.collect_logits(session.step, steps)
     assert {(source[rid], p) for rid, p in got} == {k for k in want if k[0] in set(source.values())}
     worst = compare(got, want, source.get, LIMIT[dtype])
-    print(f"7B layer sizes, 2 layers, {rows} rows decoding, graphs={graphs}, {dtype}: worst relative error {worst:.3e}")
+    print(f"real layer sizes, {rows} rows decoding, graphs={graphs}, {dtype}: worst relative error {worst:.3e}")
     if graphs:
         assert session.runner.graph_replays == 32
         widest = max(b for b, c in session.runner.graphs)
         assert widest >= rows and (rows <= 16 or widest > 16)
+    assert session.cache.all_free()
+
+
+def test_tuned_library_products_match_plain(oracles):
+    """With the library's kernels for a full prompt portion chosen by measurement, as the benchmark
+    and serving run them, whole prompts in bfloat16 still give the plain logits: the chosen kernels
+    are compared with the plain implementation, not with the engine's untuned self."""
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.replay import TraceSession
+    d, reqs, want, _ = oracles(S7)
+    model, _ = load_model(d, "bfloat16", "cuda:0")
+    searched = model.tune_library(len(reqs["long"]))       # the row count of the step that is compared
+    assert searched >= 4, "q/k/v, o, gate/up and down were to be searched"
+    steps = only_kept(helpers.steps_whole({"long": reqs["long"], "mid": reqs["mid"]}))
+    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=PAGE)
+    got = helpers.collect_logits(session.step, steps)
+    worst = compare(got, want, limit=LIMIT["bfloat16"])
+    print(f"7B layer sizes, tuned library products, whole prompts, bfloat16: worst relative error {worst:.3e}")
     assert session.cache.all_free()

@@ -224,3 +224,93 @@ def test_massive_hidden_channels_keep_the_tolerance(name, dtype, tmp_path):
         session = TraceSession(model, helpers.max_live_tokens(steps), page_size=helpers.PAGE[name])
         worst = _compare(helpers.collect_logits(session.step, steps), want, reqs, LIMIT[dtype])
         print(f"config {name} with massive channels, {cut}, {dtype}: worst relative error {worst:.3e}")
+
+
+LONG_TOKENS, LONG_PORTION, LONG_TAIL = 8192 + 33, 2048, 64
+
+
+@pytest.fixture(scope="module", params=["B", "D"])
+def long_case(request, tmp_path_factory):
+    """One request of 8,225 tokens.  With weights as random as the others' every key would weigh about
+    1/8000 and a run of keys left out or taken twice would hide in the tolerance, so the query and key
+    projections are four times as large: the scores spread over a few units and a fraction of the keys,
+    anywhere among the thousands, carries each position's sum.  (Six times as large, and the rounding
+    of the bfloat16 scores alone, 2^-9 of a score of ten, takes the logits to the bfloat16 limit.)"""
+    import torch
+    from safetensors.torch import load_file, save_file
+    name = request.param
+    d = helpers.make_model_dir(tmp_path_factory, name, seed=31)
+    path = os.path.join(d, "model.safetensors")
+    t = load_file(path)
+    for k in list(t):
+        if k.endswith(("q_proj.weight", "k_proj.weight")):
+            t[k] = (t[k].to(torch.float32) * 4).to(t[k].dtype)
+    save_file(t, path, metadata={"format": "pt"})
+    w, cfg = plain.load_folder(d)
+    toks = helpers.prompts_for(name, [LONG_TOKENS], seed=13)[0]
+    with torch.inference_mode():
+        logits = plain.model_forward(w, cfg, toks)
+    first_decoded = LONG_TOKENS - LONG_TAIL
+    kept = sorted({min(s + LONG_PORTION, first_decoded) - 1 for s in range(0, first_decoded, LONG_PORTION)}
+                  | set(range(first_decoded, LONG_TOKENS)))
+    return name, d, toks, {p: logits[p].numpy().copy() for p in kept}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_context_in_portions_then_decoded_across_a_graph_bucket_matches_plain(long_case, dtype):
+    """A context of more than 8,192 tokens as a whole model against the plain implementation: the
+    prompt in portions of 2,048 (prompt attention behind thousands of cached keys), the last 64
+    tokens decoded one by one from graphs, across the edge between the context buckets of 8,192 and
+    of the pool's size, where decode attention's key splits change their length."""
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.replay import TraceSession
+    name, d, toks, want = long_case
+    first_decoded = LONG_TOKENS - LONG_TAIL
+    steps = []
+    for s in range(0, first_decoded, LONG_PORTION):
+        n = min(LONG_PORTION, first_decoded - s)
+        steps.append({"entries": [{"id": "long", "tokens": toks[s:s + n], "want": [n - 1]}], "end": []})
+    for p in range(first_decoded, LONG_TOKENS):
+        steps.append({"entries": [{"id": "long", "tokens": [toks[p]], "want": [0]}], "end": ["long"] if p == LONG_TOKENS - 1 else []})
+    model, _ = load_model(d, dtype, "cuda:0")
+    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=helpers.PAGE[name], max_requests=2, graphs=True)
+    got = helpers.collect_logits(session.step, steps)
+    assert {p for _, p in got} == set(want)
+    scale = max(float(np.abs(row).max()) for row in want.values())
+    worst = 0.0
+    for (_, p), row in got.items():
+        err = float(np.abs(row - want[p]).max()) / scale
+        assert np.isfinite(err) and err < LIMIT[dtype], f"position {p}: relative error {err:.3e} >= {LIMIT[dtype]}"
+        worst = max(worst, err)
+    print(f"config {name}, {LONG_TOKENS} tokens, {dtype}: worst relative error {worst:.3e}")
+    assert session.runner.graph_replays == LONG_TAIL
+    assert {c for _, c in session.runner.graphs} == {8192, session.runner.fit_context}, "both context buckets were to replay"
+    assert session.cache.all_free()
+
+
+def test_a_decoded_token_alone_and_beside_a_prompt_portion_agree_within_rounding(tmp_path):
+    """What is promised about batch mates in 32-bit: a token decoded in a step of its own and the
+    same token decoded beside another request's prompt portion are summed in different orders (the
+    attention kernel and the products choose their form from the step), so their logits are not
+    the same bits, but they differ by rounding only: both within the 32-bit limit of the plain
+    logits, and of each other."""
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.replay import TraceSession
+    for name in ("A", "B"):
+        d = helpers.make_model_dir(tmp_path / name, name, seed=8)
+        w, cfg = plain.load_folder(d)
+        a, b = helpers.prompts_for(name, [300, 45], seed=14)
+        want = plain.model_forward(w, cfg, a)[-1].numpy()
+        model, _ = load_model(d, "float32", "cuda:0")
+        rows = []
+        for beside in (False, True):
+            session = TraceSession(model, 512, page_size=helpers.PAGE[name])
+            session.step([{"id": "a", "tokens": a[:-1], "want": []}])
+            entries = [{"id": "a", "tokens": a[-1:], "want": [0]}]
+            if beside:
+                entries.insert(0, {"id": "b", "tokens": b, "want": []})
+            rows.append(session.step(entries, ["a", "b"] if beside else ["a"])[0])
+        scale = float(np.abs(want).max())
+        for row in rows:
+            assert float(np.abs(row - want).max()) / scale < LIMIT["float32"]
+        assert float(np.abs(rows[0] - rows[1]).max()) / scale < LIMIT["float32"]

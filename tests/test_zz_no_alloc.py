@@ -58,10 +58,30 @@ def test_static_argmax_matches_the_allocating_one_on_two_calls_in_a_row():
 
 def test_static_argmax_refuses_more_rows_than_its_buffer_holds():
     lib, kernels = _lib()
-    x = torch.zeros(1025, 16, device=DEV)
-    out = torch.zeros(1025, dtype=torch.int32, device=DEV)
+    g = torch.Generator(device=DEV).manual_seed(11)
+    x = torch.randn(1025, 16, device=DEV, generator=g)
+    winners = torch.arange(1025, device=DEV) % 16
+    x[torch.arange(1025, device=DEV), winners] = 9.0                     # a known winner in every row
+    out = torch.full((1025,), -1, dtype=torch.int32, device=DEV)
     assert _static(lib, x, out) != 0
     assert b"1024" in lib.tl_last_error()
+    torch.cuda.synchronize()
+    assert bool((out == -1).all()), "a refused call wrote its output"
     assert _static(lib, x[:1024], out) == 0
     torch.cuda.synchronize()
-    assert int(out.abs().sum()) == 0
+    assert torch.equal(out[:1024].long(), winners[:1024]) and int(out[1024]) == -1
+
+
+def test_static_argmax_at_its_row_limit_with_wide_rows():
+    """1,024 rows of more than 8,192 columns: the static buffer is written and read to its last
+    entry (best value and index per row and chunk), against the allocating entry point."""
+    lib, kernels = _lib()
+    g = torch.Generator(device=DEV).manual_seed(13)
+    x = torch.randn(1024, 8200, device=DEV, generator=g)
+    x[1023, 8199] = 40.0                                                 # the last row's winner in its last chunk
+    x[0, 0] = x[0, 8199] = 41.0                                          # a tie across the first and the last chunk
+    out = torch.full((1024,), -1, dtype=torch.int32, device=DEV)
+    assert _static(lib, x, out) == 0, lib.tl_last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(out, kernels.argmax(x)) and torch.equal(out.long(), x.argmax(-1))
+    assert int(out[1023]) == 8199 and int(out[0]) == 0
