@@ -427,6 +427,15 @@ __device__ __forceinline__ void am_tile_lds(const uint4* kt, const uint4* vt, in
 #define AM_VFRAG(I) vt[((((I) % DB) * 16 + c) * 8) + ((4 * ((I) / DB) + g) ^ vx)]
 #pragma unroll
     for (int i = 0; i < 4; ++i) vf[i] = AM_VFRAG(i);
+    // A vector instruction may read what a matrix-core instruction wrote only a number of cycles
+    // later, and the compiler puts that wait before instructions it knows.  The first readers of
+    // the scores below are written as assembly (am_max3), which it does not look into: so the first
+    // read is this one, of a register of each of the four last products, and nothing that follows
+    // may be moved ahead of it.
+    {
+        const float first_read = fmaxf(fmaxf(st[0][3], st[1][3]), fmaxf(st[2][3], st[3][3]));
+        asm volatile("" ::"v"(first_read));
+    }
     __builtin_amdgcn_sched_barrier(0);
     // lane (c, g) holds, of column c, keys kb + 32 h + 8 g + 4 r + i in st[2 h + r][i]
     float sv[16];

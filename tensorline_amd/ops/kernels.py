@@ -654,6 +654,22 @@ def _fit_key_splits(split_len: int, max_context: int, fit_context: int = 0) -> t
     return split_len, max(1, -(-max_context // split_len))
 
 
+def _tile32_waves(q_lens, starts, num_heads: int) -> int:
+    """Whether a step's prompt portions run on the kernel with 32 columns per wave and work-groups of
+    256 columns (8 waves; 0: no, they keep 16 columns per wave and work-groups of 128).  A work-group
+    of 256 columns reads every key tile for twice the columns, which pays where the portions' columns
+    see thousands of keys each and there are columns enough to fill the GPU with such groups;
+    measured at 28 query and 4 key/value heads of 128: a 2,048-token portion behind 30,720 cached
+    tokens 918 against 1,005 to 1,040 us, behind 14,336 492 against 500 to 530, a fresh prompt of
+    8,192 tokens 496 against 510 to 526, of 4,096 167 against 155 to 163, of 2,048 66 against 52.
+    Only the choice of kernel depends on it, never a result beyond rounding."""
+    cols = sum(n for n in q_lens if n > 1)
+    if cols == 0:
+        return 0
+    keys = sum(n * (st + (n + 1) / 2) for n, st in zip(q_lens, starts) if n > 1) / cols
+    return 8 if keys >= 4096 and cols * num_heads >= 128 * 256 else 0          # at least 128 such work-groups
+
+
 def attention_takes_head_dim(head_dim: int) -> bool:
     """The head sizes the attention kernels take: multiples of 16 up to 256 (32, 64 and 128 on the
     bfloat16 MFMA kernels, the others on the any-shape kernel)."""
@@ -677,8 +693,10 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     bfloat16 with a head size of 32, 64 or 128 and pages of a multiple of 8 tokens runs on the
     matrix cores; that kernel works per sequence and needs ``q_start`` [S+1], ``ctx_start`` [S]
     and the host-side ``plan`` (lengths of the step's sequences).  Everything else runs the
-    any-shape kernel.  ``path`` forces one: "generic", "mfma" (prompt portions on the kernel that
-    shares key tiles through LDS where the page size allows) or "mfma-direct" (independent waves);
+    any-shape kernel.  ``path`` forces one: "generic", "mfma" (prompt portions on the kernels that
+    share key tiles through LDS where the page size allows; which of the two, see ``_tile32_waves``),
+    "mfma-tile16" (16 columns per wave, work-groups of 128 columns), "mfma-tile32" (32 columns per
+    wave, work-groups of 256, head sizes 64 and 128) or "mfma-direct" (independent waves);
     ``split_keys`` forces the number of keys per split (0: no split).
 
     A step with prompt portions does not split keys: its one-token sequences would each be walked
@@ -703,7 +721,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     mfma_ok = (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and page % 8 == 0 and q_start is not None
                and ctx_start is not None and plan is not None and q_stride % 8 == 0 and o_stride % 4 == 0
                and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0)
-    if path in ("mfma", "mfma-direct"):
+    if path in ("mfma", "mfma-direct", "mfma-tile16", "mfma-tile32"):
         _check(mfma_ok, "paged_attention: the matrix-core kernel does not take these arguments")
     if mfma_ok and path != "generic":
         S = tables.shape[0]
@@ -748,6 +766,17 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if nsplit > 1:
             ws = torch.empty(T * num_heads * nsplit * (head_dim + 2), dtype=torch.float32, device=q.device)
             ws_o, ws_ml = ws[:T * num_heads * nsplit * head_dim], ws[T * num_heads * nsplit * head_dim:]
+        waves = 8 if path == "mfma-tile32" else _tile32_waves(plan.q_lens, plan.starts, num_heads) if path in (None, "mfma") else 0
+        if (waves and nt == 2 and nsplit == 1 and total128 > 0
+                and library().tl_attention_tile32_takes(head_dim, page, tables.shape[1], S, waves)):
+            # prompt portions behind many keys, head size 64 or 128: 32 columns per wave on the 32x32
+            # matrix-core instruction, work-groups of 256 columns
+            cols = 32 * waves
+            total = sum(-(-n * G // cols) for n in q_lens) + pads
+            _call("tl_attention_tile32", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
+                  _ptr(q_start), _ptr(ctx_start), _ptr(out), o_stride, T, S, num_heads, num_kv_heads, head_dim, page,
+                  int(window), ctypes.c_float(scale), waves, total, skip_single, _stream())
+            return out
         _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
               _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,
               num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,

@@ -568,11 +568,12 @@ def test_attention_prompt_tiles_page_sizes_and_long_tables(d, bs):
     each of a wave's loads lie in one page (head size x page size >= 2048) the loader works with one
     page id per load, and the values' tile in LDS is cut by pages; elsewhere with one per lane."""
     lens, q_lens = [9000, 131, 70], [300, 131, 3]
-    got, want = _attention_case(torch.bfloat16, 28, 4, d, bs, lens, q_lens, spike=True, seed=bs, path="mfma")
-    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+    for path in ("mfma-tile16", "mfma-tile32"):             # 16 columns per wave; 32 (head sizes 64 and 128, else as before)
+        got, want = _attention_case(torch.bfloat16, 28, 4, d, bs, lens, q_lens, spike=True, seed=bs, path=path)
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("path", ["generic", "mfma", "mfma-direct"])
+@pytest.mark.parametrize("path", ["generic", "mfma", "mfma-direct", "mfma-tile32"])
 @pytest.mark.parametrize("heads", [(14, 2), (12, 2), (16, 2), (4, 4), (28, 4)])
 @pytest.mark.parametrize("d", [32, 64, 128])
 def test_attention_matrix_core_kernel(path, heads, d):
@@ -614,6 +615,10 @@ def test_attention_one_token_sequences_beside_prompt_portions(heads, d, bs):
                                         spike=window == 0, route_singles=route)
             torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
             outs.append(got)
+        # the same with the portions on the kernel of 32 columns per wave
+        got, want = _attention_case(dtype, heads[0], heads[1], d, bs, lens, q_lens, window=window, seed=11,
+                                    spike=window == 0, route_singles=True, path="mfma-tile32")
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
         if window == 0:
             assert torch.equal(outs[0], outs[2])              # 5,000 keys: routed when left to choose
         portion_rows = [r for r in range(sum(q_lens)) if r not in (0, 41, 42, 343, sum(q_lens) - 1)]
@@ -774,3 +779,21 @@ def test_bad_arguments_are_refused():
         K().paged_attention(torch.randn(1, 512, device=DEV), kc, kc.permute(0, 2, 3, 1).contiguous(), torch.zeros(1, 1, dtype=torch.int32, device=DEV),
                             torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
                             1, 1, 512, 1.0)
+
+
+def test_attention_long_portions_take_the_kernel_of_32_columns_per_wave(monkeypatch):
+    """Left to choose, a long prompt portion behind thousands of keys runs on the kernel with 32
+    columns per wave and work-groups of 256 columns, a short one on that with 16 and 128; both give
+    the plain attention, a dominating far key included, and a prompt with a window too."""
+    called = []
+    call = K()._call
+    monkeypatch.setattr(K(), "_call", lambda name, *a: (called.append(name), call(name, *a))[1])
+    got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, [10000, 40], [1300, 40], spike=True, seed=4)
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+    assert called == ["tl_attention_tile32"]
+    called.clear()
+    got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, [3000, 40], [1300, 40], spike=True, seed=4)
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+    assert called == ["tl_attention_mfma"]
+    got, want = _attention_case(torch.bfloat16, 8, 2, 64, 32, [9000], [1200], window=700, seed=5, path="mfma-tile32")
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
