@@ -350,18 +350,32 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
         for (int r = 0; r < 16; ++r) acc[m][r] = 0.f;
     // Tile T into buffer BUF: nothing comes back into registers.  A key past the last one any column
     // sees is masked for every column: it is read from the place of the last keys, which stay on
-    // pages the sequence owns.
+    // pages the sequence owns.  The page ids a tile's loads need are read from LDS a step ahead
+    // (T32_PAGES), so that a wave does not start its step waiting for them.
+    int k_page[NL], v_page;
+#define T32_PAGES(T)                                                                                           \
+    {                                                                                                          \
+        const int kb_ = (T) * T32_KEYS;                                                                        \
+        int vk_ = kb_ + v_key;                                                                                 \
+        if (vk_ > khi) vk_ = khi & ~7;                                                                         \
+        v_page = tab[vk_ >> bs_shift];                                                                         \
+        _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                                       \
+            int k0_ = kb_ + (wave + i * WAVES) * KPL;                                                          \
+            if (k0_ > khi) k0_ = khi & ~(KPL - 1);                                                             \
+            k_page[i] = tab[k0_ >> bs_shift];                                                                  \
+        }                                                                                                      \
+    }
 #define T32_FETCH(T, BUF)                                                                                      \
     {                                                                                                          \
         const int kb_ = (T) * T32_KEYS;                                                                        \
         int vk_ = kb_ + v_key;                                                                                 \
         if (vk_ > khi) vk_ = khi & ~7;                                                                         \
-        const char* gv_ = v_base + (uint64_t)(uint32_t)tab[vk_ >> bs_shift] * v_stride + (vk_ & (bs - 1)) * 2; \
+        const char* gv_ = v_base + (uint64_t)(uint32_t)v_page * v_stride + (vk_ & (bs - 1)) * 2;               \
         _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                                       \
             const int L_ = wave + i * WAVES;                                                                   \
             int k0_ = kb_ + L_ * KPL;                                                                          \
             if (k0_ > khi) k0_ = khi & ~(KPL - 1);                                                             \
-            const uint32_t page_ = (uint32_t)__builtin_amdgcn_readfirstlane(tab[k0_ >> bs_shift]);            \
+            const uint32_t page_ = (uint32_t)__builtin_amdgcn_readfirstlane(k_page[i]);                       \
             const char* sk_ = kc_bytes + (uint64_t)((page_ << bs_shift) + (uint32_t)(k0_ & (bs - 1))) * k_stride; \
             t32_load_to_lds_based(sk_, k_voff, ks + (BUF) * TILE + L_ * 64);                                   \
             t32_load_to_lds(gv_ + (uint64_t)L_ * v_lstep, vs + (BUF) * TILE + L_ * 64);                        \
@@ -371,12 +385,17 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
 #define T32_LANDED() __builtin_amdgcn_s_waitcnt(0x0f70)
 
     __syncthreads();                                         // the page ids are in LDS
+    T32_PAGES(t_lo)
     T32_FETCH(t_lo, 0)
+    T32_PAGES(t_lo < t_hi ? t_lo + 1 : t_hi)
     T32_LANDED();
     __syncthreads();
     int cur = 0;
     for (int t = t_lo; t <= t_hi; ++t) {
-        if (t < t_hi) T32_FETCH(t + 1, cur ^ 1)
+        if (t < t_hi) {
+            T32_FETCH(t + 1, cur ^ 1)
+            T32_PAGES(t + 2 <= t_hi ? t + 2 : t_hi)
+        }
         const int kb = t * T32_KEYS;
         if (kb <= wk_hi && kb + T32_KEYS - 1 >= wk_lo) {     // the same for the whole wave
             const bool edge = kb + T32_KEYS - 1 > wk_full_hi || kb < wk_full_lo;
@@ -397,6 +416,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void attn_tile32_kernel(
         cur ^= 1;
     }
 #undef T32_FETCH
+#undef T32_PAGES
 #undef T32_LANDED
 
     if (!valid) return;

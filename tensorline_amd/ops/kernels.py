@@ -660,8 +660,8 @@ def _tile32_waves(q_lens, starts, num_heads: int) -> int:
     of 256 columns reads every key tile for twice the columns, which pays where the portions' columns
     see thousands of keys each and there are columns enough to fill the GPU with such groups;
     measured at 28 query and 4 key/value heads of 128: a 2,048-token portion behind 30,720 cached
-    tokens 918 against 1,005 to 1,040 us, behind 14,336 492 against 500 to 530, a fresh prompt of
-    8,192 tokens 496 against 510 to 526, of 4,096 167 against 155 to 163, of 2,048 66 against 52.
+    tokens 888 against 1,005 to 1,040 us, behind 14,336 483 against 500 to 530, a fresh prompt of
+    8,192 tokens 490 against 510 to 526, of 4,096 165 against 155 to 163, of 2,048 66 against 52.
     Only the choice of kernel depends on it, never a result beyond rounding."""
     cols = sum(n for n in q_lens if n > 1)
     if cols == 0:

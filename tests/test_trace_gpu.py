@@ -314,3 +314,51 @@ def test_a_decoded_token_alone_and_beside_a_prompt_portion_agree_within_rounding
         for row in rows:
             assert float(np.abs(row - want).max()) / scale < LIMIT["float32"]
         assert float(np.abs(rows[0] - rows[1]).max()) / scale < LIMIT["float32"]
+
+
+def test_long_portions_run_on_the_kernel_of_32_columns_per_wave_and_match_plain(tmp_path, monkeypatch):
+    """A model with 16 query heads of 64 and a request of 8,200 tokens in portions of 2,048: from the
+    third portion on (2,048 tokens behind 4,096 and more) prompt attention is given to the kernel
+    with 32 columns per wave and work-groups of 256 columns; the logits at the end of every portion
+    and at the decoded tokens are the plain ones.  Query and key projections are four times as
+    large as random ones, so that a few keys among the thousands carry each sum."""
+    import torch
+    from safetensors.torch import load_file, save_file
+    from tensorline_amd.config import Qwen2Config
+    from tensorline_amd.engine.loading import load_model
+    from tensorline_amd.engine.replay import TraceSession
+    from tensorline_amd.ops import kernels
+    from tensorline_amd.weights import write_random_model
+    cfg_dict = dict(architectures=["Qwen2ForCausalLM"], vocab_size=500, hidden_size=256, intermediate_size=384,
+                    num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=4, head_dim=64, rope_theta=1e6,
+                    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=8192)
+    d = write_random_model(Qwen2Config.from_dict(cfg_dict), str(tmp_path / "m"), seed=41)
+    path = os.path.join(d, "model.safetensors")
+    t = load_file(path)
+    for k in list(t):
+        if k.endswith(("q_proj.weight", "k_proj.weight")):
+            t[k] = (t[k].to(torch.float32) * 4).to(t[k].dtype)
+    save_file(t, path, metadata={"format": "pt"})
+    w, cfg = plain.load_folder(d)
+    total, portion, tail = 8200, 2048, 8
+    toks = [(7 * i * i + 3 * i + 1) % 500 for i in range(total)]
+    with torch.inference_mode():
+        logits = plain.model_forward(w, cfg, toks)
+    called = []
+    call = kernels._call
+    monkeypatch.setattr(kernels, "_call", lambda name, *a: (called.append(name), call(name, *a))[1])
+    first_decoded = total - tail
+    steps = []
+    for s in range(0, first_decoded, portion):
+        n = min(portion, first_decoded - s)
+        steps.append({"entries": [{"id": "r", "tokens": toks[s:s + n], "want": [0, n // 2, n - 1]}], "end": []})
+    for p in range(first_decoded, total):
+        steps.append({"entries": [{"id": "r", "tokens": [toks[p]], "want": [0]}], "end": ["r"] if p == total - 1 else []})
+    model, _ = load_model(d, "bfloat16", "cuda:0")
+    session = TraceSession(model, helpers.max_live_tokens(steps), page_size=16)
+    got = helpers.collect_logits(session.step, steps)
+    assert called.count("tl_attention_tile32") == 2 * 2, "two layers, the third and the fourth portion"
+    scale = float(logits.abs().max())
+    worst = max(float(np.abs(row - logits[p].numpy()).max()) / scale for (_, p), row in got.items())
+    print(f"16 heads of 64, {total} tokens in portions of {portion}, bfloat16: worst relative error {worst:.3e}")
+    assert worst < LIMIT["bfloat16"]
