@@ -36,16 +36,16 @@ extern "C" int tl_attention_generic(const void* q, int q_stride, const void* k_c
     const int tiles_per_seq = tl_ceil_div(max_query_len, QT);
     const long long groups = (long long)S * tiles_per_seq;
     TL_CHECK_ARG(groups <= 0x7fffffffLL, "tl_attention_generic: too many work-groups");
-    const int KT = AG_KT(d);
+    // a work-group's rows fit one wave: the waves share the keys of a tile instead (at most one token
+    // per work-group then, so that tokens are not held back by the 16-row limit: QT stays as it is)
+    const bool keys_over_waves = max_query_len * GC <= AG_WROWS && max_query_len <= QT;
+    const int KT = AG_KT(d, keys_over_waves);
     const size_t smem = ag_lds_bytes(d, KT);
     int bs_shift = -1;
     if ((bs & (bs - 1)) == 0)
         for (bs_shift = 0; (1 << bs_shift) < bs;) ++bs_shift;
     TL_CHECK_ARG(smem <= 160 * 1024, "tl_attention_generic: head size %d needs %zu bytes of LDS", d, smem);
     TL_CHECK_ARG(KT * d / 4 <= AG_MAXC * AG_THREADS, "tl_attention_generic: a tile of head size %d has too many pieces", d);
-    // a work-group's rows fit one wave: the waves share the keys of a tile instead (at most one token
-    // per work-group then, so that tokens are not held back by the 16-row limit: QT stays as it is)
-    const bool keys_over_waves = max_query_len * GC <= AG_WROWS && max_query_len <= QT;
     AgLaunch a;
     a.q = q; a.k_cache = k_cache; a.v_cache = v_cache; a.tables = tables; a.q_start = q_start; a.pos = pos; a.out = out;
     a.ws_o = ws_o; a.ws_ml = ws_ml; a.q_stride = q_stride; a.NB = NB; a.out_stride = out_stride; a.T = T;

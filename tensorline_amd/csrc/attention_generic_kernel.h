@@ -12,7 +12,7 @@
 //
 // One work-group of four waves takes up to AG_ROWS = 64 rows: the (token, query head) pairs of a run
 // of consecutive tokens of one sequence's portion and the query heads of one key/value head, a
-// wave 16 rows.  Keys are walked in tiles of KT (64, or 32 for heads above 128) that start at
+// wave 16 rows.  Keys are walked in tiles of KT (64 or 32 keys, see AG_KT) that start at
 // absolute multiples of KT.  A tile's keys and values are moved in 16-byte pieces, from the cache
 // into registers a tile ahead and from there as float into LDS: keys as [key][d], values as
 // [d][key], which is how the cache holds a page's values.  A wave computes S = Q K^T for its 16 rows
@@ -42,7 +42,10 @@
 #define AG_WROWS 16   // rows per wave
 
 #define AG_MAXC 8     // 16-byte pieces of a tile's keys (and of its values) a thread moves
-#define AG_KT(D) ((D) <= 128 ? 64 : 32)   // keys per tile for head size D
+// keys per tile for head size D: 64 up to a head size of 128 where the waves share the keys of a tile (KW),
+// 64 up to a head size of 64 otherwise; else 32, which keeps a work-group's LDS and the registers of its
+// pieces on their way small enough for two work-groups to share a CU
+#define AG_KT(D, KW) (((D) <= 64 || ((KW) && (D) <= 128)) ? 64 : 32)
 
 template <typename T>
 __device__ __forceinline__ float ag_load(const T* p) { return tl_to_float(*p); }
@@ -97,7 +100,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     T* __restrict__ out, int out_stride, int tiles_per_seq, int QT, int GC, int nq, int nkv, int bs, int bs_shift,
     int window, float scale, int nsplit, int split_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
     constexpr int d = DB * 16;
-    constexpr int KT = AG_KT(d);
+    constexpr int KT = AG_KT(d, KW);
     extern __shared__ float smem[];
     constexpr int ks_ld = d + 4;
     constexpr int vt_ld = KT + 4, ps_ld = KT + 4;

@@ -182,21 +182,30 @@ __global__ __launch_bounds__(GG_THREADS) void gemm_generic_kernel(const TA* __re
 // one output element is again summed in one fixed order that depends on K alone, not on M (1 to 16),
 // on the number of waves or on timing; it is not the order of the kernel above, whose results differ
 // from this one's by rounding.
-#define GF_SEG 512
-#ifndef GF_RING
+// Sixteen waves and segments of 256: a product with fewer tiles than the GPU has CUs (the down projection
+// of a 7B model: 224) has one work-group per CU, and what streams its weights is the loads that
+// group keeps in flight (eight waves: 2.5 TB/s for the float down projection, sixteen: 3.4), and how
+// evenly the segments deal out over the waves (74 segments of 256 over 16 waves: 5 at most, 4.6 on
+// average; 37 of 512: 3 against 2.3).  A deeper ring gains nothing (8 steps ahead: slower).
+#define GF_SEG 256
 #define GF_RING 4
-#endif
-#ifndef GF_WAVES
-#define GF_WAVES 8
-#endif
-#define GF_MAX_SEGMENTS 64    // 64 KB of LDS for the segments' sums: K up to 32,768 (beyond: the kernel above)
+#define GF_WAVES 16
+#define GF_MAX_SEGMENTS 128   // 128 KB of LDS for the segments' sums: K up to 32,768 (beyond: the kernel above)
+
+// The waves of a work-group: all sixteen where the tiles are about as many as the CUs, eight where
+// every CU holds several work-groups anyway (their loads in flight add up, and a wave with more steps
+// fills its ring less often: gate/up of a 7B model 120 against 125 us).  The result does not depend on it.
+static inline int gf_waves(int nseg, int tiles) {
+    const int most = tiles >= 512 ? GF_WAVES / 2 : GF_WAVES;
+    return nseg < most ? nseg : most;
+}
 
 // SHUF: W is the matrix-core ordered copy of a float matrix, [ceil(N/16) tiles][ceil(K/16) steps][64
 // lanes][4 values], lane 16 lg + li holding row li of the tile at k = 16 step + 4 lg .. + 4, zero
 // where it pads: a step's load of a wave is 1 KB of consecutive memory (from the row-major matrix it
 // is 16 pieces of 64 bytes, which streams at about two thirds of the rate), and needs no check.
 template <typename TA, typename TW, typename TO, bool SHUF>
-__global__ __launch_bounds__(512) void gemm_fewrows_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
+__global__ __launch_bounds__(GF_WAVES * 64) void gemm_fewrows_kernel(const TA* __restrict__ A, const TW* __restrict__ W,
                                                            const float* __restrict__ bias, TO* __restrict__ C, int M,
                                                            int N, int K, int lda, int ldc, int a_vec, int w_vec) {
     extern __shared__ float gf_part[];                       // [segment][register v][lane]
@@ -293,7 +302,7 @@ static int gg_launch(const void* A, const void* W, const float* bias, void* C, i
     } while (0)
     const int nseg = tl_ceil_div(K, GF_SEG);
     if (M <= 16 && nseg <= GF_MAX_SEGMENTS) {
-        const int waves = nseg < GF_WAVES ? nseg : GF_WAVES;
+        const int waves = gf_waves(nseg, tl_ceil_div(N, 16));
         const size_t lds = (size_t)nseg * 4 * 64 * sizeof(float);
         hipLaunchKernelGGL((gemm_fewrows_kernel<TA, TW, TO, false>), dim3(tl_ceil_div(N, 16)), dim3(64 * waves), lds, stream,
                            (const TA*)A, (const TW*)W, bias, (TO*)C, M, N, K, lda, ldc, a_vec, w_vec);
@@ -322,7 +331,7 @@ extern "C" int tl_gemm_fewrows_shuffled(const float* A, const float* Ws, const f
     if (M == 0) return 0;
     const int a_vec = ((uintptr_t)A % 16 == 0 && lda % 4 == 0) ? 1 : 0;
     const int nseg = tl_ceil_div(K, GF_SEG);
-    const int waves = nseg < GF_WAVES ? nseg : GF_WAVES;
+    const int waves = gf_waves(nseg, tl_ceil_div(N, 16));
     const size_t lds = (size_t)nseg * 4 * 64 * sizeof(float);
     hipLaunchKernelGGL((gemm_fewrows_kernel<float, float, float, true>), dim3(tl_ceil_div(N, 16)), dim3(64 * waves), lds, stream,
                        A, Ws, bias, C, M, N, K, lda, ldc, a_vec, 1);
