@@ -46,11 +46,13 @@ SHAPE_32B = dict(SHAPE_7B, hidden_size=5120, intermediate_size=27648, num_hidden
 SHAPES = {"7b": SHAPE_7B, "14b": SHAPE_14B, "32b": SHAPE_32B}
 
 
-def make_config(layers: int | None, shape: str = "7b"):
+def make_config(layers: int | None, shape: str = "7b", positions: int = 0):
     from tensorline_amd.config import Qwen2Config
     d = dict(SHAPES[shape], architectures=["Qwen2ForCausalLM"])
     if layers:
         d["num_hidden_layers"] = layers
+    if positions:
+        d["max_position_embeddings"] = positions
     return Qwen2Config.from_dict(d)
 
 
@@ -138,6 +140,48 @@ def bench_decode(llm, batch: int, context: int, steps: int, warmup: int, seed: i
         eng.abort(r)
     assert llm.cache.all_free()
     return out
+
+
+def bench_decode_at_context(llm, batch: int, context: int, steps: int, warmup: int, seed: int) -> dict:
+    """Decode steps of ``batch`` sequences at a long context without the prefill that would put them
+    there (a million tokens for 64 sequences at 16,384): every sequence is given pages for ``context``
+    tokens of a cache filled with random values, and the step function (the graphs' runner, as in
+    serving) decodes ``warmup + steps`` tokens for each, the engine's greedy pick read after every
+    step.  What a step reads and computes is what it would after a real prompt; the scheduler and the
+    overlap of its host work with the step before are not part of this measurement."""
+    import torch
+
+    from tensorline_amd.engine.batch import StepEntry
+    from tensorline_amd.ops import kernels
+    cfg, cache, runner = llm.model_config, llm.cache, llm.engine.runner
+    g = torch.Generator(device="cuda:0").manual_seed(seed)
+    for i in range(len(llm.model.schedule)):
+        if cache.owns_storage(i):
+            for plane in cache.storage(i).values():
+                plane.normal_(0.0, 0.5, generator=g)
+    first = context - (warmup + steps)
+    rids = [("long", i) for i in range(batch)]
+    for rid in rids:
+        cache.add_request(rid)
+        assert cache.grow(rid, context), "the pool is too small for this point"
+    tokens = [p[0] for p in random_prompts(batch, 1, cfg.vocab_size, seed)]
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = 0.0
+    for s in range(warmup + steps):
+        if s == warmup:
+            sync()
+            t0 = time.perf_counter()
+            e0.record()
+        logits = runner.step([StepEntry(rid, [tok], first + s, [0]) for rid, tok in zip(rids, tokens)])
+        tokens = kernels.argmax(logits).tolist()
+    e1.record()
+    sync()
+    dt = time.perf_counter() - t0
+    for rid in rids:
+        cache.release(rid)
+    assert cache.all_free()
+    return {"tok_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3, "ms_per_step_events": e0.elapsed_time(e1) / steps,
+            "mean_context": first + warmup + (steps + 1) / 2.0, "fill_s": 0.0, "graph_replays": 0}
 
 
 def bench_generate(llm, batch: int, prompt_len: int, new_tokens: int, seed: int) -> dict:
@@ -291,27 +335,22 @@ def measure_machine(dtype) -> dict:
             "gemm_TFLOPs": round(2 * n ** 3 / mm_ms / 1e9, 1)}
 
 
-def bench_workload(args) -> int:
-    """A serving-style run: many concurrent requests through the scheduler (continuous batching,
-    chunked prefill), as in the 14B and 32B workloads: ``--requests`` prompts of uniform random
-    length in [--prompt-min, --prompt-max], ``--output-tokens`` each, greedy or seeded temperature
-    sampling.  Prints one JSON line: generated tokens per second over the whole run."""
+def run_workload(llm, requests: int, prompt_min: int, prompt_max: int, output_tokens: int, temperature: float,
+                 seed: int) -> dict:
+    """``requests`` prompts of uniform random length in [prompt_min, prompt_max] given to the scheduler
+    at once (continuous batching, prompts in portions), ``output_tokens`` generated for each, greedy or
+    seeded temperature sampling; the clock runs from the call to the last token."""
     import numpy as np
     import torch
 
-    from tensorline_amd import LLM, SamplingParams
-    cfg = make_config(args.layers, args.shape)
-    rng = np.random.default_rng(args.seed)
-    lengths = rng.integers(args.prompt_min, args.prompt_max + 1, size=args.requests)
+    from tensorline_amd import SamplingParams
+    cfg = llm.model_config
+    rng = np.random.default_rng(seed)
+    lengths = rng.integers(prompt_min, prompt_max + 1, size=requests)
     prompts = [rng.integers(0, cfg.vocab_size, size=int(n)).tolist() for n in lengths]
-    max_len = args.prompt_max + args.output_tokens + 16
-    page = 16
-    llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
-              num_blocks=args.num_blocks or None, kv_mem_fraction=0.8, max_num_seqs=args.requests,
-              max_batched_tokens=2048, max_model_len=max_len, graphs=not args.no_graphs, prefix_caching=False,
-              tune_library=not args.no_tune)
-    params = [SamplingParams(max_tokens=args.output_tokens, temperature=args.temperature, top_p=1.0,
-                             stop_token_ids={-1}, seed=args.seed + i) for i in range(args.requests)]
+    params = [SamplingParams(max_tokens=output_tokens, temperature=temperature, top_p=1.0,
+                             stop_token_ids={-1}, seed=seed + i) for i in range(requests)]
+    c0 = llm.counters()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     outs = llm.generate(prompts, params)
@@ -319,22 +358,47 @@ def bench_workload(args) -> int:
     dt = time.perf_counter() - t0
     c = llm.counters()
     gen = sum(len(o.token_ids) for o in outs)
-    assert all(len(o.token_ids) == args.output_tokens for o in outs) and llm.cache.all_free()
+    assert all(len(o.token_ids) == output_tokens for o in outs) and llm.cache.all_free()
     ttft = sorted(o.stats.ttft_s for o in outs)
+    steps = c["steps"] - c0["steps"]
+    # what the run cannot do without: every step reads the weights once, every prompt token and every
+    # generated token is multiplied with them once (attention left out: a lower bound on both)
+    weight_bytes = decode_bytes(cfg, 0, 0, 2 if llm.model.dtype == torch.bfloat16 else 4)
+    flops = 2.0 * (int(lengths.sum()) + gen) * cfg.num_hidden_layers * layer_matrix_params(cfg)
+    return {"tok_s": gen / dt, "total_s": dt, "steps": steps, "prompt_tokens": int(lengths.sum()), "generated": gen,
+            "ttft_p50_s": ttft[len(ttft) // 2], "ttft_max_s": ttft[-1],
+            "preemptions": c["preemptions"] - c0["preemptions"], "graph_replays": c["graph_replays"] - c0["graph_replays"],
+            "weight_reads_GBps": steps * weight_bytes / dt / 1e9, "product_flops_per_s": flops / dt}
+
+
+def bench_workload(args) -> int:
+    """A serving-style run: many concurrent requests through the scheduler (continuous batching,
+    chunked prefill), as in the 14B and 32B workloads: ``--requests`` prompts of uniform random
+    length in [--prompt-min, --prompt-max], ``--output-tokens`` each, greedy or seeded temperature
+    sampling.  Prints one JSON line: generated tokens per second over the whole run."""
+    from tensorline_amd import LLM
+    cfg = make_config(args.layers, args.shape)
+    max_len = args.prompt_max + args.output_tokens + 16
+    page = 16
+    llm = LLM(config=cfg, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
+              num_blocks=args.num_blocks or None, kv_mem_fraction=0.8, max_num_seqs=args.requests,
+              max_batched_tokens=2048, max_model_len=max_len, graphs=not args.no_graphs, prefix_caching=False,
+              tune_library=not args.no_tune)
+    w = run_workload(llm, args.requests, args.prompt_min, args.prompt_max, args.output_tokens, args.temperature, args.seed)
     print(json.dumps({
         "metric": f"generated tok/s, {args.requests} concurrent requests (Qwen2.5-{args.shape.upper()} shape)",
-        "value": round(gen / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": c["steps"], "warmup": 0,
-        "ms_per_step": round(dt / max(c["steps"], 1) * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "value": round(w["tok_s"], 1), "unit": "tok/s", "n_gpus": 1, "steps": w["steps"], "warmup": 0,
+        "ms_per_step": round(w["total_s"] / max(w["steps"], 1) * 1e3, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype in ("bfloat16", "bf16") else "fp32",
         "data": "synthetic: random weights from a seed, token ids uniform over the vocabulary",
         "config": {"model": f"Qwen2.5-{args.shape.upper()} shape", "global_batch": args.requests, "seq_len": max_len,
                    "parallelism": "single GPU", "layers": cfg.num_hidden_layers,
                    "layers_of_shape": SHAPES[args.shape]["num_hidden_layers"], "prompt_min": args.prompt_min,
-                   "prompt_max": args.prompt_max, "output_tokens": args.output_tokens, "prompt_tokens": int(lengths.sum()),
+                   "prompt_max": args.prompt_max, "output_tokens": args.output_tokens, "prompt_tokens": w["prompt_tokens"],
                    "temperature": args.temperature, "chunk": 2048, "kv_pages": llm.cache.num_blocks, "page_size": page,
-                   "preemptions": c["preemptions"], "graph_replays": c["graph_replays"],
-                   "ttft_p50_s": round(ttft[len(ttft) // 2], 3), "ttft_max_s": round(ttft[-1], 3),
-                   "total_s": round(dt, 2)}}))
+                   "preemptions": w["preemptions"], "graph_replays": w["graph_replays"],
+                   "ttft_p50_s": round(w["ttft_p50_s"], 3), "ttft_max_s": round(w["ttft_max_s"], 3),
+                   "total_s": round(w["total_s"], 2)}}))
     return 0
 
 
@@ -443,32 +507,68 @@ def main() -> int:
         torch.cuda.empty_cache()
         sizes = {}
 
-        def other(shape: str, context: int, batch: int, steps: int):
-            c = make_config(0, shape)
-            length = context + 16
+        def other(shape: str, context: int, batch: int, steps: int, seqs: int = 0, length: int = 0, positions: int = 0,
+                  pages: int = 0):
+            """A model of all the layers of ``shape`` with room for ``seqs`` sequences of ``length`` tokens (or
+            ``pages`` pages), and its decode point at ``batch`` sequences of ``context`` tokens (none for batch 0)."""
+            c = make_config(0, shape, positions)
+            seqs, length = max(seqs, batch), max(length, context + 16)
             m = LLM(config=c, seed=args.seed, dtype=args.dtype, device="cuda:0", block_size=page,
-                    num_blocks=batch * (-(-length // page)) + 8, max_num_seqs=batch, max_batched_tokens=2048,
+                    num_blocks=pages or seqs * (-(-length // page)) + 8, max_num_seqs=seqs, max_batched_tokens=2048,
                     max_model_len=length, graphs=not args.no_graphs, graph_warmup_tokens=0, prefix_caching=False,
                     tune_library=not args.no_tune, overlap=not args.no_overlap)
+            if batch == 0:
+                return c, m, {"layers": c.num_hidden_layers}
             dec = with_roofline(bench_decode(m, batch, context, steps, 4, args.seed + 11), batch, c)
             return c, m, {"layers": c.num_hidden_layers, f"decode_b{batch}_tok_s": dec["tok_s"], f"decode_b{batch}_ms": dec["ms"],
                           f"decode_b{batch}_ctx": dec["ctx"], f"decode_b{batch}_hbm_frac": dec["hbm_frac"]}
-        for shape in ("14b", "32b"):
-            c, m, out = other(shape, args.context, 8, 16)
+
+        def portion(m, c, behind: int, tag: str) -> dict:
+            p = bench_prefill_portion(m, behind, args.prefill_tokens, 2, args.seed + 2)
+            return {f"{tag}_behind": behind, f"{tag}_tokens": args.prefill_tokens, f"{tag}_tok_s": round(p["tok_s"], 1),
+                    f"{tag}_ms": round(p["s"] * 1e3, 3),
+                    f"{tag}_frac": round(prefill_portion_flops(c, args.prefill_tokens, behind) / p["s"] / PEAK_FLOPS[dtype_key], 4)}
+
+        # the workloads the two wider shapes are quoted with: 32 requests with prompts of 256 to 4,096 tokens and
+        # 512 tokens each sampled at temperature 0.7; 64 requests of 1,024 + 256 tokens, greedy
+        workloads = {"14b": dict(requests=32, prompt_min=256, prompt_max=4096, output_tokens=512, temperature=0.7),
+                     "32b": dict(requests=64, prompt_min=1024, prompt_max=1024, output_tokens=256, temperature=0.0)}
+        for shape, wl in workloads.items():
+            c, m, out = other(shape, args.context, 8, 16, seqs=wl["requests"], length=wl["prompt_max"] + wl["output_tokens"] + 16)
             p2 = bench_prefill(m, args.prefill_tokens, 2, args.seed + 2)
             out.update({"prefill_tok_s": round(p2["tok_s"], 1), "prefill_ms": round(p2["s"] * 1e3, 3),
                         "prefill_frac": round(prefill_flops(c, args.prefill_tokens) / p2["s"] / PEAK_FLOPS[dtype_key], 4)})
+            w = run_workload(m, seed=args.seed, **wl)
+            out.update({"workload_tok_s": round(w["tok_s"], 1), "workload_requests": wl["requests"],
+                        "workload_prompt_tokens": w["prompt_tokens"], "workload_generated": w["generated"],
+                        "workload_temperature": wl["temperature"], "workload_s": round(w["total_s"], 2),
+                        "workload_steps": w["steps"], "workload_ttft_p50_s": round(w["ttft_p50_s"], 3),
+                        "workload_preemptions": w["preemptions"],
+                        # lower bounds: the weights once per step, the products of every token; attention left out
+                        "workload_hbm_frac_weights": round(w["weight_reads_GBps"] / HBM_GBPS, 4),
+                        "workload_mfma_frac_products": round(w["product_flops_per_s"] / PEAK_FLOPS[dtype_key], 4)})
             sizes[shape] = out
             del m
             gc.collect()
             torch.cuda.empty_cache()
         c, m, out = other("7b", 32768, 8, 16)
-        behind = 32768 - args.prefill_tokens
-        p3 = bench_prefill_portion(m, behind, args.prefill_tokens, 2, args.seed + 2)
-        out.update({"portion_behind": behind, "portion_tokens": args.prefill_tokens, "portion_tok_s": round(p3["tok_s"], 1),
-                    "portion_ms": round(p3["s"] * 1e3, 3),
-                    "portion_frac": round(prefill_portion_flops(c, args.prefill_tokens, behind) / p3["s"] / PEAK_FLOPS[dtype_key], 4)})
+        out.update(portion(m, c, 32768 - args.prefill_tokens, "portion"))
+        out.update(portion(m, c, 8192, "portion_8k"))
+        out.update(portion(m, c, 16384, "portion_16k"))
         sizes["7b_32k"] = out
+        del m
+        gc.collect()
+        torch.cuda.empty_cache()
+        # batch 64 at 16,384 tokens and batch 8 at 65,536 (positions beyond the shape's 32,768 allowed for this
+        # point): the cache is filled with random values instead of by a million tokens of prefill
+        points_long = ((64, 16384), (8, 65536))
+        c, m, out = other("7b", 0, 0, 0, seqs=64, length=65536 + 16, positions=131072,
+                          pages=max(b * (-(-(n + 16) // page)) for b, n in points_long) + 8)
+        out.update({"max_position_embeddings": 131072, "cache": "random values, no prefill"})
+        for batch, context in points_long:
+            d = with_roofline(bench_decode_at_context(m, batch, context, 12, 4, args.seed + 13), batch, c)
+            out.update({f"decode_b{batch}_ctx{context}_{key}": d[key] for key in ("tok_s", "ms", "ms_events", "hbm_frac")})
+        sizes["7b_long"] = out
         del m
         gc.collect()
         torch.cuda.empty_cache()
