@@ -113,6 +113,30 @@ def test_random_model_round_trip(folder):
     assert abs(float(nw.mean()) - 1.0) < 0.05 and 0.05 < float(nw.std()) < 0.15
 
 
+def test_checkpoint_tensor_names_and_shapes_are_those_of_the_reference_modules(tmp_path):
+    """The names a random model folder holds and the loader asks for, written out here: the module
+    paths the reference walks (paged.py:172-188: ``inner.embed_tokens``, ``layer.input_layernorm``,
+    ``attn.q_proj`` .. ``o_proj``, ``layer.post_attention_layernorm``, ``mlp.gate_proj`` ..
+    ``down_proj``, ``inner.norm``, ``hf.lm_head``; manager.py:52-53 for the projections' shapes), with
+    ``.weight`` and, for q/k/v, ``.bias``.  Neither side of this comparison comes from the product."""
+    cfg = Qwen2Config.from_dict(dict(architectures=["Qwen2ForCausalLM"], vocab_size=99, hidden_size=40, intermediate_size=56,
+                                     num_hidden_layers=2, num_attention_heads=6, num_key_value_heads=2, head_dim=16,
+                                     tie_word_embeddings=False))
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=1)
+    got = {name: tuple(t.shape) for name, t in load_file(os.path.join(d, "model.safetensors")).items()}
+    h, i, v, q, kv = 40, 56, 99, 6 * 16, 2 * 16
+    want = {"model.embed_tokens.weight": (v, h), "model.norm.weight": (h,), "lm_head.weight": (v, h)}
+    for layer in range(2):
+        p = f"model.layers.{layer}."
+        want.update({p + "input_layernorm.weight": (h,), p + "post_attention_layernorm.weight": (h,),
+                     p + "self_attn.q_proj.weight": (q, h), p + "self_attn.q_proj.bias": (q,),
+                     p + "self_attn.k_proj.weight": (kv, h), p + "self_attn.k_proj.bias": (kv,),
+                     p + "self_attn.v_proj.weight": (kv, h), p + "self_attn.v_proj.bias": (kv,),
+                     p + "self_attn.o_proj.weight": (h, q),
+                     p + "mlp.gate_proj.weight": (i, h), p + "mlp.up_proj.weight": (i, h), p + "mlp.down_proj.weight": (h, i)})
+    assert got == want
+
+
 def test_storage_dtypes(folder):
     d, _ = folder
     model, _ = load_model(d, "bfloat16", "cpu")
