@@ -229,7 +229,7 @@ __global__ __launch_bounds__(GF_WAVES * 64) void gemm_fewrows_kernel(const TA* _
             if (k0 >= K) {                                      // past the last segment's end: the copy ends with K
                 wv = av = make_float4(0.f, 0.f, 0.f, 0.f);
             } else {
-                wv = wtile[(size_t)(k0 / GG_KS) * 64];
+                wv = __builtin_bit_cast(float4, tl_load_stream(reinterpret_cast<const uint4*>(wtile + (size_t)(k0 / GG_KS) * 64)));
                 if (a_vec != 0 && k0 + GG_KS <= K) av = gg_load4_whole<TA>(arow_any + k0 + 4 * lg);
                 else av = gg_load4<TA>(arow, a_ok, k0 + 4 * lg, K, a_vec != 0);
             }

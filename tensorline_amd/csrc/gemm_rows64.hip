@@ -52,8 +52,8 @@ __device__ __forceinline__ void r64_issue(const bf16_t* const (&xp)[P], const ui
     for (int i = 0; i < 4; ++i) {
         int c = step * 4 + i;
         if (c > last_c) c = last_c;
-        wo[i] = w1[(size_t)c * 64];
-        if (PAIR) uo[i] = w2[(size_t)c * 64];
+        wo[i] = tl_load_stream(w1 + (size_t)c * 64);
+        if (PAIR) uo[i] = tl_load_stream(w2 + (size_t)c * 64);
     }
 }
 

@@ -161,8 +161,8 @@ __global__ __launch_bounds__(MODE == MODE_SWIGLU ? 256 : 512) void gemm_skinny_k
         for (int i = 0; i < 4; ++i) {
             int c = sc * 4 + i;
             if (c > last_c) c = last_c;
-            wf[i] = w1[(size_t)c * 64];
-            if (DUAL) uf[i] = w2[(size_t)c * 64];
+            wf[i] = tl_load_stream(w1 + (size_t)c * 64);
+            if (DUAL) uf[i] = tl_load_stream(w2 + (size_t)c * 64);
         }
     }
     for (int sc = s0; sc < s1; ++sc) {
@@ -183,8 +183,8 @@ __global__ __launch_bounds__(MODE == MODE_SWIGLU ? 256 : 512) void gemm_skinny_k
         for (int i = 0; i < 4; ++i) {
             int c = sn * 4 + i;
             if (c > last_c) c = last_c;
-            wn[i] = w1[(size_t)c * 64];
-            if (DUAL) un[i] = w2[(size_t)c * 64];
+            wn[i] = tl_load_stream(w1 + (size_t)c * 64);
+            if (DUAL) un[i] = tl_load_stream(w2 + (size_t)c * 64);
         }
         // chunks past K32 of the last step read a clamped chunk: they must count as zero
         const int cbase = sc * 4;
