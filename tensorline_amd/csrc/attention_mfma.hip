@@ -142,9 +142,6 @@ __device__ __forceinline__ int am_page_index(int k, int bs, int bs_shift) {
     return bs_shift >= 0 ? k >> bs_shift : k / bs;
 }
 
-// Keys and values of one column tile per wave (a decode step) are read once: streamed.  With more
-// column tiles the groups of a sequence read the same keys again, and they are left to the caches.
-#define AM_KV_LOAD(P) (NT == 1 ? tl_load_stream(P) : *(P))
 template <int DC, int NT>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
@@ -246,8 +243,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
         const bf16_t* kp0_ = kc + ((size_t)(p0_ * bs + k0_ - i0_ * bs) * nkv + kvh) * D + g * 8;             \
         const bf16_t* kp1_ = kc + ((size_t)(p1_ * bs + k1_ - i1_ * bs) * nkv + kvh) * D + g * 8;             \
         _Pragma("unroll") for (int dc = 0; dc < DC; ++dc) {                                                  \
-            K0[dc] = AM_KV_LOAD(reinterpret_cast<const uint4*>(kp0_ + dc * 32));                                      \
-            K1[dc] = AM_KV_LOAD(reinterpret_cast<const uint4*>(kp1_ + dc * 32));                                      \
+            K0[dc] = *reinterpret_cast<const uint4*>(kp0_ + dc * 32);                                        \
+            K1[dc] = *reinterpret_cast<const uint4*>(kp1_ + dc * 32);                                        \
         }                                                                                                    \
         int vk_ = kb_ + 8 * g;                                                                               \
         if (vk_ > khi) vk_ = khi & ~7;                                                                       \
@@ -255,7 +252,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
         const int pv_ = pages_in_lanes ? __shfl(my_page, iv_ - page_lo, TL_WAVE) : table[iv_];               \
         const bf16_t* vp_ = vc + (((size_t)pv_ * nkv + kvh) * D + c) * bs + vk_ - iv_ * bs;                  \
         _Pragma("unroll") for (int db = 0; db < DB; ++db)                                                    \
-            V[db] = AM_KV_LOAD(reinterpret_cast<const uint4*>(vp_ + (size_t)db * 16 * bs));                           \
+            V[db] = *reinterpret_cast<const uint4*>(vp_ + (size_t)db * 16 * bs);                             \
     }
     AM_LOAD_BLOCK(bb, kf0, kf1, vf)
     for (int b = bb; b < be; ++b) {

@@ -24,10 +24,11 @@ __device__ __forceinline__ uint16_t tl_f2bf_bits(float f) {
     return (uint16_t)(u >> 16);
 }
 
-// 16 bytes that are read once and not again soon (weights and cached keys and values of a decode
-// step): a non-temporal load.  Such data then does not displace what the caches hold for reuse, and
-// the long products of a decode step stream 5 to 10% faster (lm_head of a 7B model at 8 rows: 195 ->
-// 176 us, 6.2 TB/s).
+// 16 bytes that are read once and not again soon (the weights of a decode step's products): a
+// non-temporal load.  Such data then does not displace what the caches hold for reuse, and the long
+// products of a decode step stream 5 to 10% faster (lm_head of a 7B model at 8 rows: 195 -> 176 us,
+// 6.2 TB/s).  Decode attention gains nothing from it for its keys and values (batch 64) or loses
+// (batch 8: 16.4 -> 17.6 us per layer) and reads them with plain loads.
 typedef unsigned tl_u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 tl_load_stream(const uint4* p) {
     return __builtin_bit_cast(uint4, __builtin_nontemporal_load(reinterpret_cast<const tl_u32x4*>(p)));
