@@ -367,8 +367,8 @@ __global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __
     const int i8 = blockIdx.x * blockDim.x + threadIdx.x;
     if (i8 * 8 >= I) return;
     const bf16_t* row = gu + (size_t)t * 2 * I;
-    const uint4 gv = tl_load_stream(reinterpret_cast<const uint4*>(row + i8 * 8));      // read once
-    const uint4 uv = tl_load_stream(reinterpret_cast<const uint4*>(row + I + i8 * 8));
+    const uint4 gv = *reinterpret_cast<const uint4*>(row + i8 * 8);
+    const uint4 uv = *reinterpret_cast<const uint4*>(row + I + i8 * 8);
     const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
     uint32_t ow[4];
 #pragma unroll
