@@ -530,34 +530,49 @@ __device__ __forceinline__ int at_v_swizzle(int row) { return (row >> 1) & 7; }
 // the whole wave).  Written as assembly so that the compiler does not make every later LDS read wait
 // for it: a load is waited for only where AT_LANDED says so.  M0 holds the LDS base for the
 // instruction and is put back.
-__device__ __forceinline__ void at_load_to_lds(const void* g, void* lds_base) {
-    const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds_base;
+__device__ __forceinline__ void at_load_to_lds_at(const void* g, uint32_t lds_base) {
     uint32_t saved;
     asm volatile(
         "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
         : "=&s"(saved)
-        : "s"(base), "v"(g)
+        : "s"(lds_base), "v"(g)
         : "memory");
 }
+__device__ __forceinline__ void at_load_to_lds(const void* g, void* lds_base) {
+    at_load_to_lds_at(g, (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds_base);
+}
 
-template <int DC, int NT, int WAVES>
-__global__ __launch_bounds__(WAVES * 64, 32 / WAVES) void attn_tile_kernel(
+// CH = 2 ("two chains"): a work-group of twice the waves, whose second half takes every other tile of
+// the same columns, with tile buffers, running maximum, sum and accumulator of its own; at the end
+// the halves are put together through LDS as two splits of the keys are.  For steps with at most one
+// work-group per CU (a short portion behind a long context), where the longest walk sets the time and
+// a lone work-group leaves part of its CU unused.  The chains share the barrier, so they pass a
+// tile's phases together and gain less than two work-groups that drift apart would: 10 to 17%.
+template <int DC, int NT, int WAVES, int CH>
+__global__ __launch_bounds__(CH * WAVES * 64, 32 / WAVES) void attn_tile_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int32_t* __restrict__ tables, int NB, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_start, bf16_t* __restrict__ out, int out_stride, int S, int nq, int nkv, int bs,
     int bs_shift, int window, float scale, int skip_single) {
-    constexpr int THREADS = WAVES * 64;
+    constexpr int THREADS = CH * WAVES * 64;
     constexpr int WCOLS = NT * 16;                       // columns of a wave; WAVES * WCOLS = 128 per work-group
     constexpr int D = DC * 32;
     constexpr int DB = D / 16;
     constexpr int UPK = D / 8;                // uint4 per key row; also the wave-loads of a K tile and of a V^T tile
     constexpr int TILE = AT_KEYS * UPK;       // uint4 of a K tile, and of a V^T tile (D rows of 8)
     extern __shared__ uint4 at_smem[];
-    uint4* ks = at_smem;                                   // [2][TILE]
-    uint4* vs = at_smem + 2 * TILE;                        // [2][TILE]
-    int* tab = reinterpret_cast<int*>(vs + 2 * TILE);      // page ids of the sequence, as far as needed (NB ints)
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int chain = CH > 1 ? __builtin_amdgcn_readfirstlane((tid >> 6) / WAVES) : 0;
+    const int wave = (tid >> 6) - chain * WAVES;           // which 16 NT columns of the 128
+    uint4* ks = at_smem + chain * 4 * TILE;                // [2][TILE], per chain
+    uint4* vs = ks + 2 * TILE;                             // [2][TILE]
+    // with two chains: the tiles' LDS addresses for the loads, the same in every lane of a wave and said so,
+    // so that they and what is added to them stay in scalar registers
+    const uint32_t ks_lds = CH > 1 ? (uint32_t)__builtin_amdgcn_readfirstlane(
+        (int)(uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)ks) : 0u;
+    const uint32_t vs_lds = ks_lds + 2 * TILE * 16;
+    int* tab = reinterpret_cast<int*>(at_smem + CH * 4 * TILE);   // page ids of the sequence, as far as needed (NB ints)
     int* qst = tab + NB;                                   // q_start of the step (S + 1 ints)
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int kvh = blockIdx.x;                            // fastest: the heads of a group start together
     const int G = nq / nkv;
@@ -611,7 +626,7 @@ __global__ __launch_bounds__(WAVES * 64, 32 / WAVES) void attn_tile_kernel(
     int group = ngroups - 1 - flat;
     {
         const int total = (int)(gridDim.x * gridDim.y), first = AT_CUS / (int)gridDim.x;
-        if (total > AT_CUS && total <= 2 * AT_CUS && flat >= first) group = flat - first;
+        if (CH == 1 && total > AT_CUS && total <= 2 * AT_CUS && flat >= first) group = flat - first;
     }
     const int wg_col0 = group * 128;
     const int col0 = wg_col0 + wave * WCOLS;
@@ -689,11 +704,17 @@ __global__ __launch_bounds__(WAVES * 64, 32 / WAVES) void attn_tile_kernel(
             if (vk_ > khi) vk_ = khi & ~7;                                                                    \
             gv_[i] = v_base[i] + (uint64_t)(uint32_t)tab[vk_ >> bs_shift] * v_stride + (vk_ & (bs - 1)) * 2;  \
         }                                                                                                     \
+        const uint32_t buf_ = CH > 1 ? (uint32_t)__builtin_amdgcn_readfirstlane((BUF) * TILE * 16) : 0u;      \
         _Pragma("unroll") for (int i = 0; i < NI; ++i) {                                                      \
             const int w_ = wave_u + i * WAVES;                                                                \
             if (w_ < UPK) {                                                                                   \
-                at_load_to_lds(gk_[i], ks + (BUF) * TILE + w_ * 64);                                          \
-                at_load_to_lds(gv_[i], vs + (BUF) * TILE + w_ * 64);                                          \
+                if (CH > 1) {                                                                                 \
+                    at_load_to_lds_at(gk_[i], ks_lds + buf_ + w_ * 1024);                                     \
+                    at_load_to_lds_at(gv_[i], vs_lds + buf_ + w_ * 1024);                                     \
+                } else {                                                                                      \
+                    at_load_to_lds(gk_[i], ks + (BUF) * TILE + w_ * 64);                                      \
+                    at_load_to_lds(gv_[i], vs + (BUF) * TILE + w_ * 64);                                      \
+                }                                                                                             \
             }                                                                                                 \
         }                                                                                                     \
     }
@@ -701,29 +722,83 @@ __global__ __launch_bounds__(WAVES * 64, 32 / WAVES) void attn_tile_kernel(
 #define AT_LANDED() __builtin_amdgcn_s_waitcnt(0x0f70)
 
     __syncthreads();                                         // the page ids are in LDS
-    AT_FETCH(t_lo, 0)
-    AT_LANDED();
-    __syncthreads();
+#define AT_TILE(T)                                                                                             \
+    {                                                                                                         \
+        const uint4* kt = ks + cur * TILE;                                                                    \
+        const uint4* vt = vs + cur * TILE;                                                                    \
+        if (NT == 1 && (T) * AT_KEYS + 32 <= wk_hi && (T) * AT_KEYS + 31 >= wk_lo) {                          \
+            /* both halves hold keys of the wave: the whole tile at once */                                   \
+            am_tile_lds<DC>(kt, vt, kx, vx, qf[0], p_col[0], lo_col[0], (T) * AT_KEYS, c, g, scale2, m_run[0], \
+                            l_run[0], acc[0]);                                                                \
+        } else {                                                                                              \
+            _Pragma("unroll") for (int half = 0; half < 2; ++half) {                                          \
+                const int kb = (T) * AT_KEYS + half * 32;                                                     \
+                if (kb > wk_hi || kb + 31 < wk_lo) continue; /* the same for the whole wave */                \
+                am_block_lds<DC, NT>(kt, vt, kx, vx, half, qf, p_col, lo_col, kb, c, g, scale2, m_run, l_run, acc); \
+            }                                                                                                 \
+        }                                                                                                     \
+    }
     int cur = 0;
-    for (int t = t_lo; t <= t_hi; ++t) {
-        if (t < t_hi) AT_FETCH(t + 1, cur ^ 1)
-        const uint4* kt = ks + cur * TILE;
-        const uint4* vt = vs + cur * TILE;
-        if (NT == 1 && t * AT_KEYS + 32 <= wk_hi && t * AT_KEYS + 31 >= wk_lo) {
-            // both halves hold keys of the wave: the whole tile at once
-            am_tile_lds<DC>(kt, vt, kx, vx, qf[0], p_col[0], lo_col[0], t * AT_KEYS, c, g, scale2, m_run[0], l_run[0],
-                            acc[0]);
-        } else {
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int kb = t * AT_KEYS + half * 32;
-                if (kb > wk_hi || kb + 31 < wk_lo) continue;  // the same for the whole wave
-                am_block_lds<DC, NT>(kt, vt, kx, vx, half, qf, p_col, lo_col, kb, c, g, scale2, m_run, l_run, acc);
-            }
-        }
+    if (CH == 1) {
+        AT_FETCH(t_lo, 0)
         AT_LANDED();
         __syncthreads();
-        cur ^= 1;
+        for (int t = t_lo; t <= t_hi; ++t) {
+            if (t < t_hi) AT_FETCH(t + 1, cur ^ 1)
+            AT_TILE(t)
+            AT_LANDED();
+            __syncthreads();
+            cur ^= 1;
+        }
+    } else {
+        // chain c takes tiles t_lo + c, t_lo + c + CH, ...; every wave passes the same barriers, a chain
+        // whose tile lies past the last one loads that one again and computes nothing
+        const int iters = (t_hi - t_lo + CH) / CH;
+        int t = t_lo + chain;
+        AT_FETCH((t <= t_hi ? t : t_hi), 0)
+        AT_LANDED();
+        __syncthreads();
+        for (int it = 0; it < iters; ++it, t += CH) {
+            if (it + 1 < iters) AT_FETCH((t + CH <= t_hi ? t + CH : t_hi), cur ^ 1)
+            if (t <= t_hi) AT_TILE(t)
+            AT_LANDED();
+            __syncthreads();
+            cur ^= 1;
+        }
+    }
+#undef AT_TILE
+
+    if (CH > 1) {
+        // The second chain hands its running maximum, sum and accumulator over through LDS (the tiles
+        // are done with: every wave has passed the last barrier), lane to lane: the same lane of the
+        // same wave number holds the same columns and dims in both chains.
+        constexpr int PER = DB * 4 + 2;
+        float* hand = reinterpret_cast<float*>(at_smem) + (size_t)wave * NT * PER * 64 + lane;
+        if (chain == 1) {
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                hand[(j * PER + 0) * 64] = m_run[j];
+                hand[(j * PER + 1) * 64] = l_run[j];
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) hand[(j * PER + 2 + db * 4 + i) * 64] = acc[j][db][i];
+            }
+        }
+        __syncthreads();
+        if (chain == 1) return;                              // no barrier follows
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const float m1 = hand[(j * PER + 0) * 64], l1 = hand[(j * PER + 1) * 64];
+            const float mm = fmaxf(m_run[j], m1);            // base-2 domain, as in the loop
+            const float w0 = (m_run[j] > -INFINITY) ? exp2f(m_run[j] - mm) : 0.f;
+            const float w1 = (m1 > -INFINITY) ? exp2f(m1 - mm) : 0.f;
+            l_run[j] = l_run[j] * w0 + l1 * w1;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[j][db][i] = acc[j][db][i] * w0 + hand[(j * PER + 2 + db * 4 + i) * 64] * w1;
+        }
     }
 
 #pragma unroll
@@ -750,8 +825,8 @@ __global__ __launch_bounds__(WAVES * 64, 32 / WAVES) void attn_tile_kernel(
 // LDS of the tile kernel for head size 32 * DC, a table of `pages` page ids and S sequences: 64 KB of tiles at
 // head size 128, so two work-groups share a CU's 160 KB up to some 8,000 pages per sequence and one
 // work-group has it alone beyond that
-static size_t at_lds_bytes(int DC, int pages, int S) {
-    return (size_t)(4 * AT_KEYS * DC * 4) * sizeof(uint4) + (size_t)(pages + S + 1) * sizeof(int);
+static size_t at_lds_bytes(int DC, int pages, int S, int chains = 1) {
+    return (size_t)chains * (4 * AT_KEYS * DC * 4) * sizeof(uint4) + (size_t)(pages + S + 1) * sizeof(int);
 }
 
 // Merge the splits of one (token, head): M = max m_s, out = sum acc_s e^(m_s - M) / sum l_s e^(m_s - M),
@@ -918,16 +993,25 @@ extern "C" int tl_attention_mfma(const void* q, int q_stride, const void* k_cach
     const bool pow2 = (bs & (bs - 1)) == 0;
     if (NT == 2 && nsplit == 1 && shared && pow2 && !seq_list && total_groups128 > 0 &&
         at_lds_bytes(d / 32, NB, S) <= 160 * 1024) {
-        // 128 columns per work-group, keys and values shared through LDS
+        // 128 columns per work-group, keys and values shared through LDS; shared == 2 asks for two
+        // chains per work-group where their tiles fit LDS
         int bs_shift = 0;
         while ((1 << bs_shift) < bs) ++bs_shift;
         TL_CHECK_ARG(total_groups128 <= 65535, "tl_attention_mfma: %d column groups are more than a launch takes", total_groups128);
         dim3 sgrid(nkv, (unsigned)total_groups128, 1);
-        const size_t lds = at_lds_bytes(d / 32, NB, S);
+        const int chains = (shared == 2 && at_lds_bytes(d / 32, NB, S, 2) <= 160 * 1024) ? 2 : 1;
+        const size_t lds = at_lds_bytes(d / 32, NB, S, chains);
 #define TL_TILE_CASE(DCV)                                                                                             \
-    hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT>), sgrid, dim3(64 * 8 / AT_NT), lds, stream, qq,        \
-                       q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, S, nq, nkv, bs,     \
-                       bs_shift, window, scale, skip_single)
+    do {                                                                                                              \
+        if (chains == 2)                                                                                              \
+            hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT, 2>), sgrid, dim3(2 * 64 * 8 / AT_NT), lds,    \
+                               stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, \
+                               S, nq, nkv, bs, bs_shift, window, scale, skip_single);                                 \
+        else                                                                                                          \
+            hipLaunchKernelGGL((attn_tile_kernel<DCV, AT_NT, 8 / AT_NT, 1>), sgrid, dim3(64 * 8 / AT_NT), lds,        \
+                               stream, qq, q_stride, kk, vv, tables, NB, q_start, ctx_start, (bf16_t*)out, out_stride, \
+                               S, nq, nkv, bs, bs_shift, window, scale, skip_single);                                 \
+    } while (0)
         if (d == 32) TL_TILE_CASE(1);
         else if (d == 64) TL_TILE_CASE(2);
         else TL_TILE_CASE(4);

@@ -654,6 +654,22 @@ def _fit_key_splits(split_len: int, max_context: int, fit_context: int = 0) -> t
     return split_len, max(1, -(-max_context // split_len))
 
 
+def _tile16_chains(total128: int, num_kv_heads: int, path) -> int:
+    """1 or 2: whether a work-group of the 16-columns-per-wave prompt kernel walks its keys as one
+    chain of tiles or as two that take every other tile (twice the waves, put together at the end).
+    Two where there is at most one work-group per CU: then the longest walk sets the time, and the
+    second chain uses what a lone work-group leaves of its CU (1,024 tokens behind 4,096 at the 7B
+    shape: 107 -> 96 us, 512 behind 8,192: 158 -> 131, 64 behind 3,000: 57 -> 50).  With more
+    work-groups than CUs two of one chain per CU do as well or better (the two chains of a work-group
+    pass their tiles' phases together, two work-groups drift apart and overlap them): a fresh prompt
+    of 2,048 tokens takes 51 us either way, one of 3,072 94 against 113."""
+    if path == "mfma-tile16x2":
+        return 2
+    if path == "mfma-tile16":
+        return 1
+    return 2 if total128 * num_kv_heads <= 256 else 1
+
+
 def _tile32_waves(q_lens, starts, num_heads: int) -> int:
     """Whether a step's prompt portions run on the kernel with 32 columns per wave and work-groups of
     256 columns (8 waves; 0: no, they keep 16 columns per wave and work-groups of 128).  A work-group
@@ -695,7 +711,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     and the host-side ``plan`` (lengths of the step's sequences).  Everything else runs the
     any-shape kernel.  ``path`` forces one: "generic", "mfma" (prompt portions on the kernels that
     share key tiles through LDS where the page size allows; which of the two, see ``_tile32_waves``),
-    "mfma-tile16" (16 columns per wave, work-groups of 128 columns), "mfma-tile32" (32 columns per
+    "mfma-tile16" (16 columns per wave, work-groups of 128 columns walking their keys as one chain of
+    tiles; "mfma-tile16x2": as two chains), "mfma-tile32" (32 columns per
     wave, work-groups of 256, head sizes 64 and 128) or "mfma-direct" (independent waves);
     ``split_keys`` forces the number of keys per split (0: no split).
 
@@ -721,7 +738,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     mfma_ok = (q.dtype == torch.bfloat16 and head_dim in (32, 64, 128) and page % 8 == 0 and q_start is not None
                and ctx_start is not None and plan is not None and q_stride % 8 == 0 and o_stride % 4 == 0
                and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0)
-    if path in ("mfma", "mfma-direct", "mfma-tile16", "mfma-tile32"):
+    if path in ("mfma", "mfma-direct", "mfma-tile16", "mfma-tile16x2", "mfma-tile32"):
         _check(mfma_ok, "paged_attention: the matrix-core kernel does not take these arguments")
     if mfma_ok and path != "generic":
         S = tables.shape[0]
@@ -780,7 +797,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
               _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,
               num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,
-              0 if path == "mfma-direct" else 1, total128, _ptr(None), 0, skip_single, _stream())
+              0 if path == "mfma-direct" else _tile16_chains(total128, num_kv_heads, path), total128, _ptr(None), 0,
+              skip_single, _stream())
         return out
     # The any-shape kernel tiles each sequence's tokens: it needs the first row of every sequence and the
     # most tokens one of them brings.  The engine has both; a bare call derives them from seq_of_token.

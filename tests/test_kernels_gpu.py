@@ -568,12 +568,13 @@ def test_attention_prompt_tiles_page_sizes_and_long_tables(d, bs):
     each of a wave's loads lie in one page (head size x page size >= 2048) the loader works with one
     page id per load, and the values' tile in LDS is cut by pages; elsewhere with one per lane."""
     lens, q_lens = [9000, 131, 70], [300, 131, 3]
-    for path in ("mfma-tile16", "mfma-tile32"):             # 16 columns per wave; 32 (head sizes 64 and 128, else as before)
+    # 16 columns per wave, one chain of tiles per work-group and two; 32 (head sizes 64 and 128, else as before)
+    for path in ("mfma-tile16", "mfma-tile16x2", "mfma-tile32"):
         got, want = _attention_case(torch.bfloat16, 28, 4, d, bs, lens, q_lens, spike=True, seed=bs, path=path)
         torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("path", ["generic", "mfma", "mfma-direct", "mfma-tile32"])
+@pytest.mark.parametrize("path", ["generic", "mfma", "mfma-direct", "mfma-tile16x2", "mfma-tile32"])
 @pytest.mark.parametrize("heads", [(14, 2), (12, 2), (16, 2), (4, 4), (28, 4)])
 @pytest.mark.parametrize("d", [32, 64, 128])
 def test_attention_matrix_core_kernel(path, heads, d):
@@ -797,3 +798,22 @@ def test_attention_long_portions_take_the_kernel_of_32_columns_per_wave(monkeypa
     assert called == ["tl_attention_mfma"]
     got, want = _attention_case(torch.bfloat16, 8, 2, 64, 32, [9000], [1200], window=700, seed=5, path="mfma-tile32")
     torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+
+
+def test_attention_short_portions_behind_long_contexts_walk_their_keys_as_two_chains(monkeypatch):
+    """Left to choose, a step with at most one work-group of 128 columns per CU asks the prompt
+    kernel for two chains of tiles per work-group, a step with more for one; both give the plain
+    attention where one far key dominates, with an odd number of tiles (the second chain has one
+    fewer), a single tile (it has none), a window, and a one-token sequence beside the portion."""
+    asked = []
+    call = K()._call
+    monkeypatch.setattr(K(), "_call", lambda name, *a: (asked.append((name, a[25] if len(a) > 25 else None)), call(name, *a))[1])
+    for lens, q_lens, window in (([4200, 40], [300, 40], 0), ([2900, 1], [64, 1], 0), ([60], [33], 0), ([5000], [500], 700)):
+        asked.clear()
+        got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, lens, q_lens, window=window, spike=True, seed=6)
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+        assert asked == [("tl_attention_mfma", 2)], asked
+    asked.clear()
+    got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, [3000, 40], [1300, 40], spike=True, seed=4)
+    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+    assert asked == [("tl_attention_mfma", 1)], asked
