@@ -950,7 +950,8 @@ static void launch_attn(int NT, dim3 grid, int wg_waves, hipStream_t stream, con
 // blocks of 32 keys, nsplit * split_blocks * 32 must cover the longest context, pos is int32 [T]
 // (the tokens' positions), ws_o holds T*nq*nsplit*d floats and ws_ml T*nq*nsplit*2.  shared != 0
 // runs unsplit steps with prompt portions on the kernel that shares keys and values through LDS
-// (when the page size and the table length allow it); shared == 0 keeps them on independent waves.
+// (when the page size and the table length allow it), shared == 2 with two chains of tiles per
+// work-group where their buffers fit; shared == 0 keeps them on independent waves.
 // A step that holds prompt portions and one-token sequences with long contexts may be run as two
 // calls: one with seq_list (int32 [n_list], the indices of one-token sequences; only they are
 // computed, with split keys, and the workspace then holds n_list rows instead of T), and one
