@@ -14,7 +14,8 @@
 // the 16x16x32 instruction feed one of 16: half the LDS traffic, half the loader's work and half
 // the per-tile bookkeeping per column, and a wave's softmax (32 exponentials and about a hundred
 // other vector instructions per tile) takes about as long as its 32 products instead of twice as
-// long.  Two work-groups of four waves share a CU (64 KB of LDS each, up to 256 registers a wave).
+// long.  A wave uses up to 256 registers, so a CU holds eight waves: one work-group of eight or two of
+// four (64 KB of LDS each).
 //
 // Operands of D = A * B (lane l: n = l % 32, h = l / 32): A is row n, eight k at 8h..8h+7; B is
 // column n, the same eight k; D register r of lane l is row 8 (r / 4) + 4 h + r % 4 of column n.
