@@ -654,7 +654,7 @@ def _fit_key_splits(split_len: int, max_context: int, fit_context: int = 0) -> t
     return split_len, max(1, -(-max_context // split_len))
 
 
-def _tile16_chains(total128: int, num_kv_heads: int, path) -> int:
+def _tile16_chains(total128: int, num_kv_heads: int, path, longest_context: int = 1 << 30) -> int:
     """1 or 2: whether a work-group of the 16-columns-per-wave prompt kernel walks its keys as one
     chain of tiles or as two that take every other tile (twice the waves, put together at the end).
     Two where there is at most one work-group per CU: then the longest walk sets the time, and the
@@ -662,12 +662,14 @@ def _tile16_chains(total128: int, num_kv_heads: int, path) -> int:
     shape: 107 -> 96 us, 512 behind 8,192: 158 -> 131, 64 behind 3,000: 57 -> 50).  With more
     work-groups than CUs two of one chain per CU do as well or better (the two chains of a work-group
     pass their tiles' phases together, two work-groups drift apart and overlap them): a fresh prompt
-    of 2,048 tokens takes 51 us either way, one of 3,072 94 against 113."""
+    of 2,048 tokens takes 51 us either way, one of 3,072 94 against 113.  Nor with walks of fewer than
+    16 tiles, where the second chain's waves and the hand-over at the end cost what they save (256
+    fresh tokens: 12.3 against 11 us)."""
     if path == "mfma-tile16x2":
         return 2
     if path == "mfma-tile16":
         return 1
-    return 2 if total128 * num_kv_heads <= 256 else 1
+    return 2 if total128 * num_kv_heads <= 256 and longest_context >= 1024 else 1
 
 
 def _tile32_waves(q_lens, starts, num_heads: int) -> int:
@@ -797,7 +799,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _call("tl_attention_mfma", _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(tables), tables.shape[1],
               _ptr(q_start), _ptr(ctx_start), _ptr(pos), _ptr(out), o_stride, _ptr(ws_o), _ptr(ws_ml), T, S, num_heads,
               num_kv_heads, head_dim, page, int(window), ctypes.c_float(scale), nt, max_groups, nsplit, split_blocks,
-              0 if path == "mfma-direct" else _tile16_chains(total128, num_kv_heads, path), total128, _ptr(None), 0,
+              0 if path == "mfma-direct" else _tile16_chains(total128, num_kv_heads, path, plan.max_context), total128,
+              _ptr(None), 0,
               skip_single, _stream())
         return out
     # The any-shape kernel tiles each sequence's tokens: it needs the first row of every sequence and the

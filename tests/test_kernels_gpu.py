@@ -801,19 +801,21 @@ def test_attention_long_portions_take_the_kernel_of_32_columns_per_wave(monkeypa
 
 
 def test_attention_short_portions_behind_long_contexts_walk_their_keys_as_two_chains(monkeypatch):
-    """Left to choose, a step with at most one work-group of 128 columns per CU asks the prompt
-    kernel for two chains of tiles per work-group, a step with more for one; both give the plain
-    attention where one far key dominates, with an odd number of tiles (the second chain has one
-    fewer), a single tile (it has none), a window, and a one-token sequence beside the portion."""
+    """Left to choose, a step with at most one work-group of 128 columns per CU and a walk of 16 tiles
+    or more asks the prompt kernel for two chains of tiles per work-group, a step with more
+    work-groups or only short walks for one; all give the plain attention where one far key
+    dominates, with an odd number of tiles (the second chain has one fewer), a window, and a
+    one-token sequence beside the portion."""
     asked = []
     call = K()._call
     monkeypatch.setattr(K(), "_call", lambda name, *a: (asked.append((name, a[25] if len(a) > 25 else None)), call(name, *a))[1])
-    for lens, q_lens, window in (([4200, 40], [300, 40], 0), ([2900, 1], [64, 1], 0), ([60], [33], 0), ([5000], [500], 700)):
+    for lens, q_lens, window in (([4200, 40], [300, 40], 0), ([2900, 1], [64, 1], 0), ([1100], [33], 0), ([5000], [500], 700)):
         asked.clear()
         got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, lens, q_lens, window=window, spike=True, seed=6)
         torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
         assert asked == [("tl_attention_mfma", 2)], asked
-    asked.clear()
-    got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, [3000, 40], [1300, 40], spike=True, seed=4)
-    torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
-    assert asked == [("tl_attention_mfma", 1)], asked
+    for lens, q_lens in (([3000, 40], [1300, 40]), ([60], [33]), ([1000, 9], [700, 9])):
+        asked.clear()
+        got, want = _attention_case(torch.bfloat16, 28, 4, 128, 16, lens, q_lens, spike=True, seed=4)
+        torch.testing.assert_close(got, want, atol=2e-2, rtol=2e-2)
+        assert asked == [("tl_attention_mfma", 1)], asked
